@@ -1,0 +1,51 @@
+"""The tensors behind the cache manager's ids.
+
+A paged group has one pool [caches in group, 2 (k, v), num_pages, KV, block_size, D]
+in the compute dtype: the block_size keys of one head in one page are contiguous.  It
+starts zeroed, so that no slot ever holds a non-finite value
+(reference atomserve/kv_cache.py:112-118).  A state group has
+[caches in group, max_num_seqs, *shape].
+"""
+
+import torch
+
+from atomserve_amd.cache.manager import CacheManager
+
+
+class CachePools:
+    def __init__(self, manager: CacheManager, dtype: torch.dtype, device):
+        self.manager = manager
+        self.dtype = dtype
+        self.paged = []
+        for g in manager.paged_groups:
+            r = g.request
+            shape = (len(g.cache_ids), 2, manager.num_blocks, r.num_kv_heads, manager.block_size, r.head_dim)
+            self.paged.append(torch.zeros(shape, dtype=dtype, device=device))
+        self.state = []
+        for g in manager.state_groups:
+            shape = (len(g.cache_ids), manager.max_num_seqs, *g.request.shape)
+            self.state.append(torch.zeros(shape, dtype=g.request.dtype, device=device))
+
+    def pages(self, cache_id: int):
+        """(group index, k_pages, v_pages) of one cache; views [num_pages, KV, block_size, D]."""
+        kind, gi, li = self.manager.group_of_cache[cache_id]
+        if kind != "paged":
+            raise KeyError(f"cache {cache_id} is not paged")
+        return gi, self.paged[gi][li, 0], self.paged[gi][li, 1]
+
+    def state_of(self, cache_id: int):
+        """(group index, state tensor [max_num_seqs, *shape]) of one cache."""
+        kind, gi, li = self.manager.group_of_cache[cache_id]
+        if kind != "state":
+            raise KeyError(f"cache {cache_id} holds no fixed-size state")
+        return gi, self.state[gi][li]
+
+    @staticmethod
+    def bytes_per_block(requests: dict, block_size: int, dtype: torch.dtype) -> int:
+        """Memory one page id costs across all paged caches, keys and values
+        (reference atomserve/kv_cache.py:129-135)."""
+        from atomserve_amd.parts.base import PagedCacheRequest
+
+        item = torch.empty((), dtype=dtype).element_size()
+        return sum(2 * r.num_kv_heads * r.head_dim * item * block_size
+                   for r in requests.values() if isinstance(r, PagedCacheRequest))  # fmt: skip

@@ -1,0 +1,274 @@
+// Attention over the paged cache.
+//
+// Cache pages of one layer: k_pages, v_pages [num_pages, KV, block_size, D]; a token
+// at position p of a request lives in page table[p / block_size] at offset
+// p % block_size.  A query at position p sees the keys at positions lo..p, with
+// lo = max(0, p - window + 1) if window > 0, else 0.  Query head h reads kv head
+// h / (H / KV).  Scores, softmax and the weighted sum are fp32.
+//
+// attn_single_query: one work item per query token.  A workgroup (4 waves) takes one
+// token, one kv head, up to GT query heads of its group, and one partition of
+// `part_size` keys.  Inside a wave, LPK lanes share a key (each holds 16 bytes of
+// the head) and 64 / LPK keys are in flight at once, each such lane group keeping an
+// online-softmax stream (m, l, acc) of its own; streams are merged by shuffles, waves
+// through LDS, partitions by attn_reduce.  Serves fp32 (every row) and bf16 (decode).
+// Plain reference: reference atomserve/kernels.py:167-334, atomserve/model.py:269-289.
+#include "common.h"
+
+#define NEG_INF (-__builtin_inff())
+
+template <typename T> struct Chunk;  // 16 bytes of a head
+template <> struct Chunk<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 r = *reinterpret_cast<const float4*>(p);
+    v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+  }
+};
+template <> struct Chunk<bf16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const bf16* p, float* v) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+
+template <typename T, int GT>
+__global__ __launch_bounds__(256) void attn_single_query_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    const int* __restrict__ items, const int* __restrict__ positions, const int* __restrict__ tok_row,
+    const int* __restrict__ block_tables, int table_width, T* __restrict__ out,
+    float* __restrict__ part_m, float* __restrict__ part_l, float* __restrict__ part_acc, int H, int KV,
+    int D, int bs, float scale, int window, int part_size, int P, int lpk) {
+  constexpr int CH = Chunk<T>::N;
+  extern __shared__ float smem[];  // [4][GT] m, [4][GT] l, [4][GT][D] acc
+  const int G = H / KV;
+  const int HC = (G + GT - 1) / GT;
+  const int item = blockIdx.x, kvh = blockIdx.y / HC, hc = blockIdx.y % HC, part = blockIdx.z;
+  const int t = items[item];
+  const int pos = positions[t];
+  const int ctx = pos + 1;
+  const int lo = window > 0 ? max(0, ctx - window) : 0;
+  const int k0 = max(lo, part * part_size), k1 = min(ctx, (part + 1) * part_size);
+  const int h0 = kvh * G + hc * GT;       // first query head of this workgroup
+  const int ng = min(GT, G - hc * GT);    // valid heads among the GT
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  if (k0 >= k1) {  // an empty partition (P > 1 only): mark it so for the reduce
+    if (tid < ng) {
+      const size_t o = ((size_t)item * H + h0 + tid) * P + part;
+      part_m[o] = NEG_INF;
+      part_l[o] = 0.f;
+    }
+    return;
+  }
+
+  const int nsub = 64 / lpk;  // keys in flight per wave
+  const int sub = lane / lpk, j = lane % lpk;
+  const bool active = j * CH < D;
+  const int* table = block_tables + (size_t)tok_row[t] * table_width;
+
+  float qr[GT][CH];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    if (active && g < ng) {
+      Chunk<T>::load(q + ((size_t)t * H + h0 + g) * D + j * CH, qr[g]);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) qr[g][c] *= scale;
+    } else {
+#pragma unroll
+      for (int c = 0; c < CH; ++c) qr[g][c] = 0.f;
+    }
+  }
+
+  float m[GT], l[GT], acc[GT][CH];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    m[g] = NEG_INF;
+    l[g] = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) acc[g][c] = 0.f;
+  }
+
+  const int stride = 4 * nsub;
+  const int iters = (k1 - k0 + stride - 1) / stride;  // uniform over the workgroup
+  for (int it = 0; it < iters; ++it) {
+    const int key = k0 + it * stride + wave * nsub + sub;
+    const bool valid = key < k1;
+    float kv[CH], vv[CH];
+    if (valid && active) {
+      const int page = table[key / bs];
+      const size_t base = (((size_t)page * KV + kvh) * bs + key % bs) * D + j * CH;
+      Chunk<T>::load(k_pages + base, kv);
+      Chunk<T>::load(v_pages + base, vv);
+    } else {
+#pragma unroll
+      for (int c = 0; c < CH; ++c) { kv[c] = 0.f; vv[c] = 0.f; }
+    }
+    float s[GT];
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      float d = 0.f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) d += qr[g][c] * kv[c];
+      for (int off = 1; off < lpk; off <<= 1) d += __shfl_xor(d, off, WAVE);
+      s[g] = d;
+    }
+    if (valid) {
+#pragma unroll
+      for (int g = 0; g < GT; ++g) {
+        const float mn = fmaxf(m[g], s[g]);
+        const float a = __expf(m[g] - mn);  // m = -inf gives 0
+        const float p = __expf(s[g] - mn);
+        l[g] = l[g] * a + p;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) acc[g][c] = acc[g][c] * a + p * vv[c];
+        m[g] = mn;
+      }
+    }
+  }
+
+  // merge the streams of a wave
+  for (int off = lpk; off < 64; off <<= 1) {
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      const float mo = __shfl_xor(m[g], off, WAVE), lo_ = __shfl_xor(l[g], off, WAVE);
+      const float mn = fmaxf(m[g], mo);
+      const float a = (m[g] == NEG_INF) ? 0.f : __expf(m[g] - mn);
+      const float b = (mo == NEG_INF) ? 0.f : __expf(mo - mn);
+      l[g] = l[g] * a + lo_ * b;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const float ao = __shfl_xor(acc[g][c], off, WAVE);
+        acc[g][c] = acc[g][c] * a + ao * b;
+      }
+      m[g] = mn;
+    }
+  }
+
+  float* sm = smem;
+  float* sl = smem + 4 * GT;
+  float* sacc = smem + 8 * GT;
+  if (lane < lpk) {
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      if (j == 0) { sm[wave * GT + g] = m[g]; sl[wave * GT + g] = l[g]; }
+      if (active) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) sacc[((size_t)wave * GT + g) * D + j * CH + c] = acc[g][c];
+      }
+    }
+  }
+  __syncthreads();
+
+  for (int idx = tid; idx < ng * D; idx += 256) {
+    const int g = idx / D, d = idx % D;
+    float mx = NEG_INF;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, sm[w * GT + g]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = sm[w * GT + g];
+      const float e = (mw == NEG_INF) ? 0.f : __expf(mw - mx);
+      num += sacc[((size_t)w * GT + g) * D + d] * e;
+      den += sl[w * GT + g] * e;
+    }
+    const int h = h0 + g;
+    if (P == 1) {
+      out[((size_t)t * H + h) * D + d] = from_f32<T>(num / den);
+    } else {
+      const size_t o = ((size_t)item * H + h) * P + part;
+      part_acc[o * D + d] = num;
+      if (d == 0) { part_m[o] = mx; part_l[o] = den; }
+    }
+  }
+}
+
+// Merge the partitions of each (item, head): out = sum_p acc_p e^(m_p - M) / sum_p l_p e^(m_p - M).
+template <typename T>
+__global__ void attn_reduce_kernel(const int* __restrict__ items, const float* __restrict__ part_m,
+                                   const float* __restrict__ part_l, const float* __restrict__ part_acc,
+                                   T* __restrict__ out, int H, int D, int P) {
+  const int item = blockIdx.x, h = blockIdx.y;
+  const size_t o = ((size_t)item * H + h) * P;
+  float mx = NEG_INF;
+  for (int p = 0; p < P; ++p) mx = fmaxf(mx, part_m[o + p]);
+  float den = 0.f;
+  for (int p = 0; p < P; ++p) {
+    const float mp = part_m[o + p];
+    den += (mp == NEG_INF) ? 0.f : part_l[o + p] * __expf(mp - mx);
+  }
+  const int t = items[item];
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float num = 0.f;
+    for (int p = 0; p < P; ++p) {
+      const float mp = part_m[o + p];
+      if (mp != NEG_INF) num += part_acc[(o + p) * D + d] * __expf(mp - mx);
+    }
+    out[((size_t)t * H + h) * D + d] = from_f32<T>(num / den);
+  }
+}
+
+static int pow2ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
+
+template <typename T>
+static int launch_single_query(const void* q, const void* k_pages, const void* v_pages, const int* items,
+                               int num_items, const int* positions, const int* tok_row,
+                               const int* block_tables, int table_width, void* out, float* part_m,
+                               float* part_l, float* part_acc, int H, int KV, int D, int bs, float scale,
+                               int window, int part_size, int P, hipStream_t stream) {
+  constexpr int CH = Chunk<T>::N;
+  if (D % CH != 0 || D > 64 * CH || D > 256) return AS_BAD_SHAPE;
+  const int G = H / KV;
+  const int lpk = pow2ceil(D / CH);
+  const int GT = G >= 8 ? 8 : (G > 2 ? 4 : (G == 2 ? 2 : 1));
+  const int HC = (G + GT - 1) / GT;
+  dim3 grid(num_items, KV * HC, P);
+  const size_t shmem = sizeof(float) * (size_t)(8 * GT + 4 * GT * D);
+#define LAUNCH(GTV)                                                                                      \
+  attn_single_query_kernel<T, GTV><<<grid, 256, shmem, stream>>>(                                        \
+      (const T*)q, (const T*)k_pages, (const T*)v_pages, items, positions, tok_row, block_tables,       \
+      table_width, (T*)out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size, P, lpk)
+  switch (GT) {
+    case 1: LAUNCH(1); break;
+    case 2: LAUNCH(2); break;
+    case 4: LAUNCH(4); break;
+    default: LAUNCH(8); break;
+  }
+#undef LAUNCH
+  if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
+  if (P > 1) {
+    attn_reduce_kernel<T><<<dim3(num_items, H), D >= 64 ? 64 : 32, 0, stream>>>(items, part_m, part_l, part_acc,
+                                                                              (T*)out, H, D, P);
+  }
+  return launch_status();
+}
+
+// part_m, part_l: [num_items, H, P] fp32; part_acc: [num_items, H, P, D] fp32 (unused when P == 1).
+// P must be >= ceil(max context of the items / part_size).
+extern "C" int as_attn_single_query(const void* q, const void* k_pages, const void* v_pages, int dtype,
+                                    const int* items, int num_items, const int* positions,
+                                    const int* tok_row, const int* block_tables, int table_width, void* out,
+                                    float* part_m, float* part_l, float* part_acc, int H, int KV, int D,
+                                    int bs, float scale, int window, int part_size, int P,
+                                    hipStream_t stream) {
+  if (num_items <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || H % KV || D <= 0 || bs <= 0 || part_size <= 0 || P <= 0 || table_width <= 0)
+    return AS_BAD_SHAPE;
+  if (P > 1 && (!part_m || !part_l || !part_acc)) return AS_BAD_SHAPE;
+  if (dtype == DT_F32)
+    return launch_single_query<float>(q, k_pages, v_pages, items, num_items, positions, tok_row, block_tables,
+                                      table_width, out, part_m, part_l, part_acc, H, KV, D, bs, scale,
+                                      window, part_size, P, stream);
+  if (dtype == DT_BF16)
+    return launch_single_query<bf16>(q, k_pages, v_pages, items, num_items, positions, tok_row, block_tables,
+                                     table_width, out, part_m, part_l, part_acc, H, KV, D, bs, scale, window,
+                                     part_size, P, stream);
+  return AS_BAD_DTYPE;
+}

@@ -1,0 +1,224 @@
+// Row-wise kernels of the decoder: embedding lookup, RMSNorm with the residual sum
+// fused in, the rotary table, per-head q/k norm + rotation + cache store, and the
+// gated activation.  All arithmetic is fp32; storage is fp32 or bf16.
+#include "common.h"
+
+// ---- embedding --------------------------------------------------------------------
+// out[t, :] = table[ids[t], :] as fp32 (the residual stream is always fp32).
+// Plain reference: reference atomserve/model.py:373.
+template <typename T>
+__global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, int width, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // ids are validated on the host; never read outside
+  const T* src = table + (size_t)id * width;
+  float* dst = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+extern "C" int as_embed_gather(const void* table, int table_dtype, const int* ids, float* out,
+                               int num_tokens, int width, int vocab, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (width <= 0 || vocab <= 0) return AS_BAD_SHAPE;
+  const int threads = width >= 1024 ? 256 : 64;
+  if (table_dtype == DT_F32)
+    embed_gather_kernel<float><<<num_tokens, threads, 0, stream>>>((const float*)table, ids, out, width, vocab);
+  else if (table_dtype == DT_BF16)
+    embed_gather_kernel<bf16><<<num_tokens, threads, 0, stream>>>((const bf16*)table, ids, out, width, vocab);
+  else
+    return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- RMSNorm with fused residual sum and row selection --------------------------
+// For output row r (source row s = rows ? rows[r] : r):
+//   v = x[s] + (delta ? delta[s] : 0)          in fp32; written back to x[s] if update_x
+//   out[r] = v / sqrt(mean(v^2) + eps) * w     rounded once
+// Plain reference: reference atomserve/model.py:125-139 (weight multiplies directly).
+template <typename O, typename W>
+__global__ void rmsnorm_kernel(float* __restrict__ x, const O* __restrict__ delta,
+                               const int* __restrict__ rows, const W* __restrict__ w, float eps,
+                               O* __restrict__ out, int n, int update_x) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = x + s * n;
+  const O* dr = delta ? delta + s * n : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) {
+      v += to_f32(dr[i]);
+      if (update_x) xr[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  O* o = out + (size_t)r * n;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];  // the thread's own earlier store, if any, is what it reads back
+    if (dr && !update_x) v += to_f32(dr[i]);
+    o[i] = from_f32<O>(v * inv * to_f32(w[i]));
+  }
+}
+
+extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const void* w, int w_dtype,
+                          float eps, void* out, int out_dtype, int num_out_rows, int n, int update_x,
+                          hipStream_t stream) {
+  if (num_out_rows <= 0) return AS_OK;
+  if (n <= 0) return AS_BAD_SHAPE;
+  const int threads = n >= 2048 ? 256 : (n >= 512 ? 128 : 64);
+#define LAUNCH(O, W)                                                                              \
+  rmsnorm_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)delta, rows, (const W*)w, \
+                                                             eps, (O*)out, n, update_x)
+  if (out_dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (out_dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (out_dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- residual sum alone (the last layer's pending delta, when no norm follows) ----
+template <typename O>
+__global__ void add_delta_kernel(float* __restrict__ x, const O* __restrict__ delta, size_t count) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+    x[i] += to_f32(delta[i]);
+}
+
+extern "C" int as_add_delta(float* x, const void* delta, int delta_dtype, long count, hipStream_t stream) {
+  if (count <= 0) return AS_OK;
+  const int blocks = (int)((count + 255) / 256 > 4096 ? 4096 : (count + 255) / 256);
+  if (delta_dtype == DT_F32) add_delta_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)count);
+  else if (delta_dtype == DT_BF16) add_delta_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (size_t)count);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- rotary table -------------------------------------------------------------------
+// cs[t, i] = (cos, sin)(positions[t] * inv_freq[i]), i < half.  The product and the
+// range reduction are done in fp64 so that large positions keep fp32-exact angles;
+// the rotation itself is fp32.  Plain reference: reference atomserve/model.py:142-169.
+__global__ void rope_table_kernel(const int* __restrict__ positions, const double* __restrict__ inv_freq,
+                                  float2* __restrict__ cs, int num_tokens, int half) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= num_tokens * half) return;
+  const int t = idx / half, i = idx % half;
+  const double a = (double)positions[t] * inv_freq[i];
+  double s, c;
+  sincos(a, &s, &c);
+  cs[idx] = make_float2((float)c, (float)s);
+}
+
+extern "C" int as_rope_table(const int* positions, const double* inv_freq, float* cs, int num_tokens,
+                             int half, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (half <= 0) return AS_BAD_SHAPE;
+  const int total = num_tokens * half;
+  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, (float2*)cs, num_tokens, half);
+  return launch_status();
+}
+
+// ---- per-head q/k norm + rotation + cache store -----------------------------------
+// One wave per (token, head slot) of qkv [T, H + 2 KV, D].  q and k heads: optional
+// RMSNorm over the head's D values with gains qw / kw, then rotation of the pairs
+// (i, i + R/2), i < R/2, by the token's angle; coordinates >= R pass unrotated.
+// q goes to q_out [T, H, D]; k and v go to the cache pages [num_pages, KV, bs, D] at
+// slot = page * bs + offset.  v is copied as it is.  store_kv = 0 computes q only.
+// Plain reference: reference atomserve/kernels.py:74-145, atomserve/model.py:326-333.
+template <typename O, typename W>
+__global__ void qk_norm_rope_store_kernel(const O* __restrict__ qkv, const W* __restrict__ qw,
+                                          const W* __restrict__ kw, const float2* __restrict__ cs,
+                                          const int* __restrict__ slots, O* __restrict__ q_out,
+                                          O* __restrict__ k_pages, O* __restrict__ v_pages, int H, int KV,
+                                          int D, int R, float eps, int block_size) {
+  const int t = blockIdx.x, hs = blockIdx.y, lane = threadIdx.x;
+  const O* src = qkv + ((size_t)t * (H + 2 * KV) + hs) * D;
+  const bool is_q = hs < H, is_k = !is_q && hs < H + KV;
+  O* dst;
+  if (is_q) {
+    dst = q_out + ((size_t)t * H + hs) * D;
+  } else {
+    const int slot = slots[t];
+    if (slot < 0) return;  // this token's keys are not stored (whole wave returns)
+    const int kvh = is_k ? hs - H : hs - H - KV;
+    O* pages = is_k ? k_pages : v_pages;
+    dst = pages + (((size_t)(slot / block_size) * KV + kvh) * block_size + slot % block_size) * D;
+  }
+  if (!is_q && !is_k) {
+    for (int i = lane; i < D; i += WAVE) dst[i] = src[i];
+    return;
+  }
+  const W* w = is_q ? qw : kw;
+  float inv = 1.0f;
+  if (w) {
+    float ss = 0.f;
+    for (int i = lane; i < D; i += WAVE) { const float v = to_f32(src[i]); ss += v * v; }
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)D + eps);
+  }
+  const int half = R / 2;
+  for (int i = lane; i < half; i += WAVE) {
+    float a = to_f32(src[i]) * inv, b = to_f32(src[i + half]) * inv;
+    if (w) { a *= to_f32(w[i]); b *= to_f32(w[i + half]); }
+    float c = 1.f, s = 0.f;
+    if (cs) { const float2 v = cs[(size_t)t * half + i]; c = v.x; s = v.y; }
+    dst[i] = from_f32<O>(a * c - b * s);
+    dst[i + half] = from_f32<O>(b * c + a * s);
+  }
+  for (int i = R + lane; i < D; i += WAVE) {
+    float a = to_f32(src[i]) * inv;
+    if (w) a *= to_f32(w[i]);
+    dst[i] = from_f32<O>(a);
+  }
+}
+
+extern "C" int as_qk_norm_rope_store(const void* qkv, int dtype, const void* qw, const void* kw, int w_dtype,
+                                     const float* cs, const int* slots, void* q_out, void* k_pages,
+                                     void* v_pages, int num_tokens, int H, int KV, int D, int R, float eps,
+                                     int block_size, int store_kv, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || D <= 0 || R < 0 || R > D || (R & 1) || block_size <= 0) return AS_BAD_SHAPE;
+  if ((qw == nullptr) != (kw == nullptr)) return AS_BAD_SHAPE;
+  dim3 grid(num_tokens, store_kv ? H + 2 * KV : H);
+#define LAUNCH(O, W)                                                                                   \
+  qk_norm_rope_store_kernel<O, W><<<grid, WAVE, 0, stream>>>(                                          \
+      (const O*)qkv, (const W*)qw, (const W*)kw, (const float2*)cs, slots, (O*)q_out, (O*)k_pages,    \
+      (O*)v_pages, H, KV, D, R, eps, block_size)
+  if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- gated activation -----------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g / (1 + exp(-g)).
+// Plain reference: reference atomserve/kernels.py:439-449, atomserve/model.py:358-359.
+template <typename O>
+__global__ void silu_mul_kernel(const O* __restrict__ gu, O* __restrict__ out, int inter, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inter;
+    const int i = (int)(idx % inter);
+    const float g = to_f32(gu[t * 2 * inter + i]);
+    const float u = to_f32(gu[t * 2 * inter + inter + i]);
+    out[idx] = from_f32<O>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int as_silu_mul(const void* gate_up, void* out, int dtype, int num_tokens, int inter,
+                           hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (inter <= 0) return AS_BAD_SHAPE;
+  const size_t total = (size_t)num_tokens * inter;
+  const size_t want = (total + 255) / 256;
+  const int blocks = (int)(want > 8192 ? 8192 : want);
+  if (dtype == DT_F32) silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter, total);
+  else if (dtype == DT_BF16) silu_mul_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, inter, total);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}

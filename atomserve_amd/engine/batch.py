@@ -1,0 +1,203 @@
+"""A step's work, flattened: rows of (request, next tokens) become flat integer arrays,
+uploaded in one copy (reference atomserve/runner.py:87-158, 215-241).
+
+A `Row` says: these tokens, at positions start.., for the request whose pages are
+these tables; logits are wanted at these places among them.  Everything before `start`
+is already in the cache.  Rows of any length mix freely in one step.
+"""
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from atomserve_amd.cache.manager import RELEASED
+
+TILE_Q = 64  # query tokens per work item of the prefill attention kernel
+SHORT_ROW = 8  # rows up to this many tokens are attended as single queries (reference runner.py:31-34)
+
+
+@dataclass
+class Row:
+    """tokens: the new tokens, at positions start, start + 1, ...
+    tables: the request's block table in each paged group; must cover every new position
+    want:   indices into `tokens` whose next-token logits are asked for
+    state_slot: the request's slot in the fixed-size state tables, or -1
+    """
+
+    tokens: list
+    start: int
+    tables: list
+    want: list = field(default_factory=list)
+    state_slot: int = -1
+
+
+def slot_of(block_table: list, position: int, block_size: int) -> int:
+    """Pool slot of the token at `position` (reference atomserve/runner.py:37-39)."""
+    return block_table[position // block_size] * block_size + position % block_size
+
+
+class _View:
+    pass
+
+
+class PagedLayerView(_View):
+    """What an attention mixer sees of its cache in one step."""
+
+    __slots__ = ("k_pages", "v_pages", "slots", "block_tables", "writes", "block_size")
+
+    def __init__(self, k_pages, v_pages, slots, block_tables, writes, block_size):
+        self.k_pages, self.v_pages, self.slots, self.block_tables = k_pages, v_pages, slots, block_tables
+        self.writes, self.block_size = writes, block_size
+
+
+class StateLayerView(_View):
+    """What a mixer with fixed-size state sees: its state table and each row's slot."""
+
+    __slots__ = ("state", "row_slots", "writes")
+
+    def __init__(self, state, row_slots, writes):
+        self.state, self.row_slots, self.writes = state, row_slots, writes
+
+
+class StepBatch:
+    """The flat batch of one step, on the device.
+
+    token_ids, positions, tok_row [T] int32   (tok_row: which row a token belongs to)
+    logits_rows [B'] int32                    flat indices of the wanted positions
+    group_slots[g] [T], group_tables[g] [R, W_g] int32, per paged group
+    all_tokens [T]; short_tokens [Ns]: tokens of rows with <= SHORT_ROW tokens;
+    long_tiles [Nt, 4]: (first flat token, count, row, first position) per TILE_Q queries of longer rows
+    row_first, row_len, row_start, row_slots [R] int32 (for mixers with per-request state)
+    """
+
+    def __init__(self, rows, block_size: int, num_paged_groups: int, vocab_size: int, device, pools=None,
+                 staging=None):  # fmt: skip
+        if not rows:
+            raise ValueError("a step needs at least one row")
+        bs = block_size
+        tok, pos, trow, want = [], [], [], []
+        slots = [[] for _ in range(num_paged_groups)]
+        short, tiles = [], []
+        row_first, row_len, row_start, row_slots = [], [], [], []
+        widths = [1] * num_paged_groups
+        flat = 0
+        self.max_context = self.max_short_context = 0
+        for r, row in enumerate(rows):
+            n, end = len(row.tokens), row.start + len(row.tokens)
+            if n < 1 or row.start < 0:
+                raise ValueError(f"bad row: {n} tokens at position {row.start}")
+            if any(not 0 <= w < n for w in row.want):
+                raise ValueError(f"bad row: wanted places {row.want} outside its {n} tokens")
+            bad = [t for t in row.tokens if not 0 <= t < vocab_size]
+            if bad:
+                raise ValueError(f"token id {bad[0]} is outside the vocabulary of {vocab_size}")
+            if len(row.tables) != num_paged_groups:
+                raise ValueError(f"row has {len(row.tables)} block tables, the model has {num_paged_groups} groups")
+            for g, table in enumerate(row.tables):
+                if end > len(table) * bs:
+                    raise ValueError(f"block table holds {len(table) * bs} slots, need {end}")
+                first_page, last_page = row.start // bs, (end - 1) // bs
+                if any(table[b] == RELEASED for b in range(first_page, last_page + 1)):
+                    raise ValueError("block table has given back a page that this row writes")
+                slots[g].extend(table[p // bs] * bs + p % bs for p in range(row.start, end))
+                widths[g] = max(widths[g], (end + bs - 1) // bs)
+            tok.extend(row.tokens)
+            pos.extend(range(row.start, end))
+            trow.extend([r] * n)
+            want.extend(flat + w for w in row.want)
+            if n <= SHORT_ROW:
+                short.extend(range(flat, flat + n))
+                self.max_short_context = max(self.max_short_context, end)
+            else:
+                for q0 in range(0, n, TILE_Q):
+                    tiles.extend((flat + q0, min(TILE_Q, n - q0), r, row.start + q0))
+            self.max_context = max(self.max_context, end)
+            row_first.append(flat)
+            row_len.append(n)
+            row_start.append(row.start)
+            row_slots.append(row.state_slot)
+            flat += n
+
+        T, R = flat, len(rows)
+        tables = []
+        for g in range(num_paged_groups):
+            w = widths[g]
+            arr = np.zeros((R, w), dtype=np.int32)
+            for r, row in enumerate(rows):
+                t = row.tables[g][:w]
+                arr[r, : len(t)] = [0 if p == RELEASED else p for p in t]
+            tables.append(arr)
+
+        fields = [("token_ids", tok), ("positions", pos), ("tok_row", trow), ("logits_rows", want),
+                  ("all_tokens", range(T)), ("short_tokens", short), ("long_tiles", tiles),
+                  ("row_first", row_first), ("row_len", row_len), ("row_start", row_start),
+                  ("row_slots", row_slots)]  # fmt: skip
+        for g in range(num_paged_groups):
+            fields.append((f"slots{g}", slots[g]))
+            fields.append((f"tables{g}", tables[g].reshape(-1)))
+        arrays = [np.asarray(list(v) if not isinstance(v, np.ndarray) else v, dtype=np.int32) for _, v in fields]
+        total = sum(a.size for a in arrays)
+        if staging is not None:
+            host = staging.take(total)
+        else:
+            host = torch.empty(total, dtype=torch.int32, pin_memory=torch.device(device).type == "cuda")
+        np.concatenate(arrays, out=host.numpy()[:total]) if total else None
+        dev = host[:total].to(device, non_blocking=True)
+        if staging is not None:
+            staging.sent()
+        self._host = host  # alive until the copy has run
+        offset, parts = 0, {}
+        for (name, _), a in zip(fields, arrays):
+            parts[name] = dev[offset : offset + a.size]
+            offset += a.size
+
+        self.num_tokens, self.num_rows = T, R
+        self.token_ids, self.positions, self.tok_row = parts["token_ids"], parts["positions"], parts["tok_row"]
+        self.logits_rows, self.num_logits = parts["logits_rows"], len(want)
+        self.all_tokens = parts["all_tokens"]
+        self.short_tokens, self.num_short_tokens = parts["short_tokens"], len(short)
+        self.long_tiles, self.num_long_tiles = parts["long_tiles"].view(-1, 4), len(tiles) // 4
+        self.row_first, self.row_len = parts["row_first"], parts["row_len"]
+        self.row_start, self.row_slots = parts["row_start"], parts["row_slots"]
+        self.group_slots = [parts[f"slots{g}"] for g in range(num_paged_groups)]
+        self.group_tables = [parts[f"tables{g}"].view(R, widths[g]) for g in range(num_paged_groups)]
+        self.host_rows = rows
+        self.block_size = bs
+        self.pools = pools
+        self.shared = {}  # per-step results that parts share (rotary tables, ...)
+
+    def cache_view(self, cache_id: int, writes: bool):
+        """The view of cache `cache_id` for a mixer in this step."""
+        kind, gi, _ = self.pools.manager.group_of_cache[cache_id]
+        if kind == "paged":
+            _, k_pages, v_pages = self.pools.pages(cache_id)
+            return PagedLayerView(k_pages, v_pages, self.group_slots[gi], self.group_tables[gi], writes, self.block_size)
+        _, state = self.pools.state_of(cache_id)
+        return StateLayerView(state, self.row_slots, writes)
+
+
+class Staging:
+    """Two pinned host buffers used in turn for the step uploads; a buffer is reused only after
+    the copy that read it has run."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.buffers = [None, None]
+        self.events = [None, None]
+        self.turn = 0
+
+    def take(self, count: int):
+        i = self.turn
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        if self.buffers[i] is None or self.buffers[i].numel() < count:
+            self.buffers[i] = torch.empty(max(count, 4096), dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        return self.buffers[i]
+
+    def sent(self) -> None:
+        if self.device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            self.events[self.turn] = ev
+        self.turn ^= 1

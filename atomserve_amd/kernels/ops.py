@@ -1,0 +1,244 @@
+"""One checked Python wrapper per HIP kernel.
+
+Each wrapper verifies on the host what the kernel and its grid assume (device, dtype,
+contiguity, shapes) and only then launches on torch's current stream.  Nothing here
+computes with torch operators: if a library is missing the call raises.
+"""
+
+import math
+
+import torch
+
+from atomserve_amd.kernels.lib import KernelError, call
+
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+_DT = {F32: 0, BF16: 1}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(t, name, dtype=None, shape=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name} must be a tensor on the GPU")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None:
+        allowed = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
+        if t.dtype not in allowed:
+            raise KernelError(f"{name} has dtype {t.dtype}, expected {allowed}")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and int(d) != int(s) for d, s in zip(t.shape, shape)):
+            raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def embed_gather(table, ids, out) -> None:
+    """out[t] = table[ids[t]] as fp32.  table [V, h] fp32|bf16, ids [T] int32, out [T, h] fp32."""
+    _check(table, "table", (F32, BF16), (None, None))
+    vocab, width = table.shape
+    _check(ids, "ids", I32, (None,))
+    _check(out, "out", F32, (ids.shape[0], width))
+    call("as_embed_gather", _ptr(table), _DT[table.dtype], _ptr(ids), _ptr(out), ids.shape[0], width, vocab, _stream())
+
+
+def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True) -> None:
+    """out[r] = norm(x[s] + delta[s]) * weight with s = rows[r] (or r); x fp32 [T, n] gets the
+    sum written back when `delta` is given and `update_x`.  out, delta: fp32|bf16."""
+    _check(x, "x", F32, (None, None))
+    T, n = x.shape
+    _check(weight, "weight", (F32, BF16), (n,))
+    n_out = T
+    if rows is not None:
+        _check(rows, "rows", I32, (None,))
+        n_out = rows.shape[0]
+    _check(out, "out", (F32, BF16), (n_out, n))
+    if delta is not None:
+        _check(delta, "delta", out.dtype, (T, n))
+    if out.dtype == F32 and weight.dtype != F32:
+        raise KernelError("fp32 norm needs an fp32 weight")
+    call("as_rmsnorm", _ptr(x), _ptr(delta), _ptr(rows), _ptr(weight), _DT[weight.dtype], float(eps), _ptr(out),
+         _DT[out.dtype], n_out, n, int(bool(update_x)), _stream())  # fmt: skip
+
+
+def add_delta(x, delta) -> None:
+    """x += delta (x fp32, delta fp32|bf16, same shape)."""
+    _check(x, "x", F32)
+    _check(delta, "delta", (F32, BF16), tuple(x.shape))
+    call("as_add_delta", _ptr(x), _ptr(delta), _DT[delta.dtype], x.numel(), _stream())
+
+
+def rope_table(positions, inv_freq, out) -> None:
+    """out[t, i] = (cos, sin)(positions[t] * inv_freq[i]); inv_freq fp64 [R/2], out fp32 [T, R/2, 2]."""
+    _check(positions, "positions", I32, (None,))
+    _check(inv_freq, "inv_freq", torch.float64, (None,))
+    _check(out, "out", F32, (positions.shape[0], inv_freq.shape[0], 2))
+    call("as_rope_table", _ptr(positions), _ptr(inv_freq), _ptr(out), positions.shape[0], inv_freq.shape[0], _stream())
+
+
+def qk_norm_rope_store(qkv, q_weight, k_weight, cos_sin, slots, q_out, k_pages, v_pages, num_heads,
+                       num_kv_heads, eps, store_kv=True) -> None:  # fmt: skip
+    """Per-head norm (if weights are given), rotation (if `cos_sin` is given) and the cache store.
+
+    qkv [T, H + 2 KV, D]; q_out [T, H, D]; pages [num_pages, KV, block_size, D]; slots [T] int32
+    (page * block_size + offset, or -1 for a token whose keys are not stored)."""
+    _check(qkv, "qkv", (F32, BF16), (None, num_heads + 2 * num_kv_heads, None))
+    T, _, D = qkv.shape
+    _check(q_out, "q_out", qkv.dtype, (T, num_heads, D))
+    R = 0
+    if cos_sin is not None:
+        _check(cos_sin, "cos_sin", F32, (T, None, 2))
+        R = 2 * cos_sin.shape[1]
+        if R > D:
+            raise KernelError(f"rotary width {R} exceeds head width {D}")
+    w_dtype = qkv.dtype
+    if q_weight is not None:
+        _check(q_weight, "q_weight", (F32, BF16), (D,))
+        _check(k_weight, "k_weight", q_weight.dtype, (D,))
+        w_dtype = q_weight.dtype
+        if qkv.dtype == F32 and w_dtype != F32:
+            raise KernelError("fp32 q/k norm needs fp32 weights")
+    elif k_weight is not None:
+        raise KernelError("q and k norm weights come together")
+    block_size = 1
+    if store_kv:
+        _check(slots, "slots", I32, (T,))
+        _check(k_pages, "k_pages", qkv.dtype, (None, num_kv_heads, None, D))
+        _check(v_pages, "v_pages", qkv.dtype, tuple(k_pages.shape))
+        block_size = k_pages.shape[2]
+    call("as_qk_norm_rope_store", _ptr(qkv), _DT[qkv.dtype], _ptr(q_weight), _ptr(k_weight), _DT[w_dtype],
+         _ptr(cos_sin), _ptr(slots) if store_kv else 0, _ptr(q_out), _ptr(k_pages) if store_kv else 0,
+         _ptr(v_pages) if store_kv else 0, T, num_heads, num_kv_heads, D, R, float(eps), block_size,
+         int(bool(store_kv)), _stream())  # fmt: skip
+
+
+def silu_mul(gate_up, out) -> None:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _check(gate_up, "gate_up", (F32, BF16), (None, None))
+    T, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError("gate_up needs an even width")
+    _check(out, "out", gate_up.dtype, (T, two_i // 2))
+    call("as_silu_mul", _ptr(gate_up), _ptr(out), _DT[gate_up.dtype], T, two_i // 2, _stream())
+
+
+SINGLE_QUERY_MAX_HEAD_DIM = 256
+
+
+def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tables, out, scale, window,
+                      max_context, part_size=None) -> None:  # fmt: skip
+    """Attention of single query tokens over the paged cache.
+
+    q, out [T, H, D]; items [N] int32: the tokens (rows of q) to process; positions, tok_row [T]
+    int32; block_tables [R, W] int32; max_context: host bound on positions[items] + 1."""
+    _check(q, "q", (F32, BF16), (None, None, None))
+    T, H, D = q.shape
+    _check(out, "out", q.dtype, (T, H, D))
+    _check(k_pages, "k_pages", q.dtype, (None, None, None, D))
+    _check(v_pages, "v_pages", q.dtype, tuple(k_pages.shape))
+    _, KV, bs, _ = k_pages.shape
+    _check(items, "items", I32, (None,))
+    _check(positions, "positions", I32, (T,))
+    _check(tok_row, "tok_row", I32, (T,))
+    _check(block_tables, "block_tables", I32, (None, None))
+    N = items.shape[0]
+    if N == 0:
+        return
+    chunk = 4 if q.dtype == F32 else 8
+    if H % KV or D % chunk or D > SINGLE_QUERY_MAX_HEAD_DIM:
+        raise KernelError(f"attention: unsupported heads {H}/{KV} or head width {D} "
+                          f"(needs a multiple of {chunk}, at most {SINGLE_QUERY_MAX_HEAD_DIM})")  # fmt: skip
+    if max_context > block_tables.shape[1] * bs:
+        raise KernelError("attention: block tables are shorter than the longest context")
+    span = min(max_context, window) if window > 0 else max_context
+    if part_size is None:
+        # Enough partitions to occupy the GPU when few tokens are in the batch, few enough
+        # that the merge stays small; boundaries are multiples of part_size in absolute position.
+        groups = N * KV * max(1, (H // KV + 7) // 8)
+        part_size = 256
+        while part_size < span and groups * math.ceil(span / part_size) > 2048:
+            part_size *= 2
+    P = max(1, math.ceil(max_context / part_size))
+    part_m = part_l = part_acc = None
+    if P > 1:
+        part_m = torch.empty((N, H, P), dtype=F32, device=q.device)
+        part_l = torch.empty((N, H, P), dtype=F32, device=q.device)
+        part_acc = torch.empty((N, H, P, D), dtype=F32, device=q.device)
+    call("as_attn_single_query", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(items), N,
+         _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m),
+         _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+
+
+def gemm(a, w, out) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T.  fp32: own kernel (true fp32).  bf16: own kernel for few
+    rows, the library's matrix product otherwise; `out` may be bf16 or (few rows) fp32."""
+    _check(a, "a", (F32, BF16), (None, None))
+    M, K = a.shape
+    _check(w, "w", a.dtype, (None, K))
+    N = w.shape[0]
+    _check(out, "out", None, (M, N))
+    if M == 0:
+        return
+    if a.dtype == F32:
+        _check(out, "out", F32)
+        call("as_gemm_f32", _ptr(a), _ptr(w), _ptr(out), M, N, K, _stream())
+        return
+    if out.dtype == BF16:
+        torch.mm(a, w.t(), out=out)
+    elif out.dtype == F32:
+        out.copy_(torch.mm(a, w.t()))
+    else:
+        raise KernelError(f"gemm: unsupported output dtype {out.dtype}")
+
+
+SAMPLE_MAX_TOP_K = 1024
+
+
+def argmax(logits, out) -> None:
+    """out[b] = index of the largest logit of row b (the lowest index among equals)."""
+    _check(logits, "logits", F32, (None, None))
+    _check(out, "out", I32, (logits.shape[0],))
+    call("as_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+
+
+def apply_penalty(logits, rows, cols, amounts) -> None:
+    """logits[rows[i], cols[i]] -= amounts[i] for distinct (row, col) pairs."""
+    _check(logits, "logits", F32, (None, None))
+    n = rows.shape[0]
+    _check(rows, "rows", I32, (n,))
+    _check(cols, "cols", I32, (n,))
+    _check(amounts, "amounts", F32, (n,))
+    call("as_apply_penalty", _ptr(logits), _ptr(rows), _ptr(cols), _ptr(amounts), n, logits.shape[1], _stream())
+
+
+def sample(logits, temperature, top_k, top_p, seeds, counters, out) -> None:
+    """One token per row: top-k (0: all), temperature (0: greedy), top-p, seeded draw.
+
+    temperature, top_p fp32 [B]; top_k, counters int32 [B]; seeds int64 [B]; out int32 [B].
+    top_k values must be 0 (or >= vocabulary) or at most SAMPLE_MAX_TOP_K; checked by the caller
+    on the host values it uploads."""
+    _check(logits, "logits", F32, (None, None))
+    B = logits.shape[0]
+    _check(temperature, "temperature", F32, (B,))
+    _check(top_k, "top_k", I32, (B,))
+    _check(top_p, "top_p", F32, (B,))
+    _check(seeds, "seeds", torch.int64, (B,))
+    _check(counters, "counters", I32, (B,))
+    _check(out, "out", I32, (B,))
+    call("as_sample", _ptr(logits), B, logits.shape[1], _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
+         _ptr(counters), _ptr(out), _stream())  # fmt: skip
+
+
+def topk(logits, k, values, indices) -> None:
+    """Sorted k largest of each row: values fp32 [B, k], indices int32 [B, k]."""
+    _check(logits, "logits", F32, (None, None))
+    B, V = logits.shape
+    if not 0 < k <= min(V, SAMPLE_MAX_TOP_K):
+        raise KernelError(f"top-k of {k} is outside 1..{min(V, SAMPLE_MAX_TOP_K)}")
+    _check(values, "values", F32, (B, k))
+    _check(indices, "indices", I32, (B, k))
+    call("as_topk", _ptr(logits), B, V, k, _ptr(values), _ptr(indices), _stream())

@@ -1,0 +1,92 @@
+"""A decoder assembled from a plan: embedding, the run list over its layers, final
+norm and head.  It knows no architecture: which parts a layer has, their sizes and
+the order of runs all come from the plan (reference atomserve/model.py:363-412 is
+the one hard-wired instance of this loop)."""
+
+import torch
+
+from atomserve_amd.kernels import ops
+from atomserve_amd.parts.base import BuildEnv, WeightDecl, build
+from atomserve_amd.parts.plan import ModelPlan
+
+
+class DecoderModel:
+    def __init__(self, plan: ModelPlan, dtype: torch.dtype, device):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"compute dtype must be float32 or bfloat16, got {dtype}")
+        self.plan = plan
+        self.env = BuildEnv(dtype=dtype, device=torch.device(device))
+        self.blocks = [build("arrangement", spec, self.env) for spec in plan.layers]
+        self.final_norm = build("norm", plan.final_norm, self.env)
+        for r in plan.run:
+            if not 0 <= r.layer < len(self.blocks):
+                raise ValueError(f"run list names layer {r.layer}, the plan has {len(self.blocks)}")
+        self.embed_weight = None
+        self.head_weight = None
+
+    # ---- tensors --------------------------------------------------------------------
+    def weight_decls(self) -> dict:
+        p = self.plan
+        decls = {"embed.weight": WeightDecl((p.vocab_size, p.hidden_size))}
+        for i, block in enumerate(self.blocks):
+            for part_name, part in block.parts().items():
+                for local, decl in part.weight_decls().items():
+                    decls[f"layers.{i}.{part_name}.{local}"] = decl
+        for local, decl in self.final_norm.weight_decls().items():
+            decls[f"final_norm.{local}"] = decl
+        if not p.tied_head:
+            decls["head.weight"] = WeightDecl((p.vocab_size, p.hidden_size))
+        return decls
+
+    def bind(self, tensors: dict) -> None:
+        """Hand every part its tensors, by the names of `weight_decls`."""
+        self.embed_weight = tensors["embed.weight"]
+        self.head_weight = self.embed_weight if self.plan.tied_head else tensors["head.weight"]
+        for i, block in enumerate(self.blocks):
+            for part_name, part in block.parts().items():
+                prefix = f"layers.{i}.{part_name}."
+                part.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+        self.final_norm.bind({k[len("final_norm."):]: v for k, v in tensors.items() if k.startswith("final_norm.")})
+        self._tensors = tensors
+
+    @property
+    def num_weight_bytes(self) -> int:
+        """Bytes of all distinct tensors (a tied head counts once)."""
+        seen = {t.data_ptr(): t.numel() * t.element_size() for t in self._tensors.values()}
+        return sum(seen.values())
+
+    # ---- caches ---------------------------------------------------------------------
+    def cache_requests(self) -> dict:
+        """cache id -> what the mixer writing it asks of the cache manager."""
+        requests = {}
+        for i, r in enumerate(self.plan.run):
+            cid = self.plan.cache_id(i)
+            req = self.blocks[r.layer].parts()["mixer"].cache_request()
+            if req is None:
+                continue
+            if r.writes:
+                if cid in requests and requests[cid] != req:
+                    raise ValueError(f"runs sharing cache {cid} ask for different caches")
+                requests[cid] = req
+        for i, r in enumerate(self.plan.run):
+            cid = self.plan.cache_id(i)
+            if self.blocks[r.layer].parts()["mixer"].cache_request() is not None and cid not in requests:
+                raise ValueError(f"run {i} reads cache {cid}, which no run writes")
+        return requests
+
+    # ---- one pass ---------------------------------------------------------------------
+    def forward(self, step) -> torch.Tensor:
+        """Run this step's tokens through every run of the plan; returns fp32 logits
+        [len(step.logits_rows), vocab] for the wanted rows."""
+        p, dev = self.plan, self.env.device
+        x = torch.empty((step.num_tokens, p.hidden_size), dtype=torch.float32, device=dev)
+        ops.embed_gather(self.embed_weight, step.token_ids, x)
+        delta = None
+        for i, r in enumerate(p.run):
+            delta = self.blocks[r.layer].forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes))
+        n = step.num_logits
+        logits = torch.empty((n, p.vocab_size), dtype=torch.float32, device=dev)
+        if n:
+            hf = self.final_norm.forward(x, delta, rows=step.logits_rows, update_residual=False)
+            ops.gemm(hf, self.head_weight, logits)
+        return logits

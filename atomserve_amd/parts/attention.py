@@ -1,0 +1,89 @@
+"""Grouped-query softmax attention over a paged cache (the mixer of this architecture).
+
+    qkv = h @ qkv_w^T;  q, k <- per-head norm (optional), rotation (optional)
+    k, v -> cache pages at the tokens' slots, written before attending
+    o = softmax(q k^T * scale over the keys a query may see) v;  out = o @ o_w^T
+
+(reference atomserve/model.py:292-336).  Every size, the scale, the window, the norm
+and the position encoding arrive through the spec.  A run that only reads another
+run's cache computes q alone and stores nothing.
+"""
+
+import torch
+
+from atomserve_amd.kernels import ops
+from atomserve_amd.parts.base import Mixer, PagedCacheRequest, WeightDecl, build, register
+
+# Rows with at most this many new tokens are attended as that many single queries
+# (reference atomserve/runner.py:31-34); longer rows go through the prefill kernel.
+SHORT_ROW = 8
+
+
+class Attention(Mixer):
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        s = spec
+        if s.num_heads % s.num_kv_heads:
+            raise ValueError(f"{s.num_heads} query heads do not divide over {s.num_kv_heads} kv heads")
+        chunk = 4 if env.dtype == torch.float32 else 8
+        if s.head_dim % chunk or s.head_dim > ops.SINGLE_QUERY_MAX_HEAD_DIM:
+            raise ValueError(
+                f"head_dim {s.head_dim} is not supported by the attention kernels "
+                f"(a multiple of {chunk}, at most {ops.SINGLE_QUERY_MAX_HEAD_DIM})"
+            )
+        self.position = build("position", s.position, env) if s.position is not None else None
+        self.q_norm_weight = self.k_norm_weight = None
+
+    def weight_decls(self) -> dict:
+        s = self.spec
+        decls = {
+            "qkv.weight": WeightDecl(((s.num_heads + 2 * s.num_kv_heads) * s.head_dim, s.hidden_size)),
+            "o.weight": WeightDecl((s.hidden_size, s.num_heads * s.head_dim)),
+        }
+        if s.qk_norm is not None:
+            decls["q_norm.weight"] = WeightDecl((s.head_dim,), role="vector")
+            decls["k_norm.weight"] = WeightDecl((s.head_dim,), role="vector")
+        return decls
+
+    def cache_request(self):
+        s = self.spec
+        return PagedCacheRequest(s.num_kv_heads, s.head_dim, s.window)
+
+    def forward(self, h, step, cache):
+        """h [T, hidden] compute dtype -> [T, hidden].  cache: a PagedLayerView (pages of this
+        run's cache, its group's slots and block tables for this step, whether to store)."""
+        s, env = self.spec, self.env
+        T = h.shape[0]
+        H, KV, D = s.num_heads, s.num_kv_heads, s.head_dim
+        qkv = torch.empty((T, (H + 2 * KV) * D), dtype=env.dtype, device=h.device)
+        ops.gemm(h, self.qkv_weight, qkv)
+        q = torch.empty((T, H, D), dtype=env.dtype, device=h.device)
+        cos_sin = self.position.prepare(step) if self.position is not None else None
+        eps = s.qk_norm.eps if s.qk_norm is not None else 0.0
+        ops.qk_norm_rope_store(
+            qkv.view(T, H + 2 * KV, D), self.q_norm_weight, self.k_norm_weight, cos_sin, cache.slots, q,
+            cache.k_pages, cache.v_pages, H, KV, eps, store_kv=cache.writes,
+        )  # fmt: skip
+        out = torch.empty((T, H, D), dtype=env.dtype, device=h.device)
+        self.attend(q, out, step, cache)
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=h.device)
+        ops.gemm(out.view(T, H * D), self.o_weight, y)
+        return y
+
+    def attend(self, q, out, step, cache) -> None:
+        s = self.spec
+        # fp32: every token is a single query.  bf16: short rows as single queries, long rows
+        # through the prefill kernel.
+        if self.env.dtype == torch.float32 or not hasattr(ops, "attn_prefill"):
+            ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
+                                  cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
+            return
+        if step.num_short_tokens:
+            ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.short_tokens, step.positions, step.tok_row,
+                                  cache.block_tables, out, s.scale, s.window, step.max_short_context)  # fmt: skip
+        if step.num_long_tiles:
+            ops.attn_prefill(q, cache.k_pages, cache.v_pages, step.long_tiles, step.positions, step.tok_row,
+                             cache.block_tables, out, s.scale, s.window)  # fmt: skip
+
+
+register("mixer", "attention", Attention)

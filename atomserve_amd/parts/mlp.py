@@ -1,0 +1,35 @@
+"""Dense gated feed-forward: down( act(gate(x)) * up(x) ) with gate and up stacked into
+one matrix (reference atomserve/model.py:339-360)."""
+
+import torch
+
+from atomserve_amd.kernels import ops
+from atomserve_amd.parts.base import FeedForward, WeightDecl, register
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        if spec.activation != "silu":
+            raise ValueError(f"activation {spec.activation!r} has no kernel (only 'silu')")
+
+    def weight_decls(self) -> dict:
+        s = self.spec
+        return {
+            "gate_up.weight": WeightDecl((2 * s.intermediate_size, s.hidden_size)),
+            "down.weight": WeightDecl((s.hidden_size, s.intermediate_size)),
+        }
+
+    def forward(self, h, step):
+        s, env = self.spec, self.env
+        T = h.shape[0]
+        gate_up = torch.empty((T, 2 * s.intermediate_size), dtype=env.dtype, device=h.device)
+        ops.gemm(h, self.gate_up_weight, gate_up)
+        act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=h.device)
+        ops.silu_mul(gate_up, act)
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=h.device)
+        ops.gemm(act, self.down_weight, y)
+        return y
+
+
+register("feed_forward", "gated_mlp", GatedMLP)

@@ -1,0 +1,3 @@
+from atomserve_amd.sampling.sampler import Sampler
+
+__all__ = ["Sampler"]

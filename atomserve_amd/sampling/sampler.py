@@ -1,0 +1,77 @@
+"""Turns next-token logits into chosen tokens, for a whole batch at once, on the GPU
+(reference atomserve/sampler.py:1-168).
+
+    logits -> presence penalty -> top-k -> / temperature -> softmax -> top-p -> draw
+
+Every row has its own settings.  A batch that is all greedy is one argmax kernel;
+otherwise one sampling kernel handles every row, greedy ones included.  The noise of
+the draw is a function of (the request's seed, how many tokens it has sampled, the
+candidate), so a request's stream does not depend on its batch neighbours; requests
+without a seed get one drawn by the engine when they are submitted.
+"""
+
+import torch
+
+from atomserve_amd.kernels import ops
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = torch.device(device)
+
+    def release(self, seq_id: int) -> None:
+        """Nothing is kept per request: the random stream is a function of the request's own
+        seed and token count (the reference keeps a generator here, sampler.py:58-60)."""
+
+    def sample(self, logits: torch.Tensor, seqs) -> list:
+        """logits [B, vocab] fp32, row i belongs to seqs[i]; returns B token ids (one host
+        synchronisation, the step's only one)."""
+        if not seqs:
+            return []
+        B, vocab = logits.shape
+        if B != len(seqs):
+            raise ValueError(f"{B} rows of logits for {len(seqs)} sequences")
+        params = [s.params for s in seqs]
+        logits = self._apply_presence_penalty(logits, seqs)
+        out = torch.empty(B, dtype=torch.int32, device=self.device)
+        if all(p.temperature == 0 for p in params):
+            ops.argmax(logits, out)
+            return out.tolist()
+        top_k = []
+        for p in params:
+            k = p.top_k if 0 < p.top_k < vocab else 0
+            if k > ops.SAMPLE_MAX_TOP_K:
+                raise ValueError(f"top_k {k} is beyond the kernel's {ops.SAMPLE_MAX_TOP_K}; use 0 for all tokens")
+            top_k.append(k)
+        floats = torch.tensor([[max(p.temperature, 0.0) for p in params], [p.top_p for p in params]],
+                              dtype=torch.float32).to(self.device, non_blocking=True)  # fmt: skip
+        ints = torch.tensor([top_k, [len(s.output_ids) for s in seqs]], dtype=torch.int32).to(self.device, non_blocking=True)
+        seeds = torch.tensor([_as_int64(s.noise_seed) for s in seqs], dtype=torch.int64).to(self.device, non_blocking=True)
+        ops.sample(logits, floats[0], ints[0], floats[1], seeds, ints[1], out)
+        return out.tolist()
+
+    def _apply_presence_penalty(self, logits, seqs):
+        """Subtract each row's penalty from the logits of the tokens it has generated so far
+        (reference atomserve/sampler.py:144-168)."""
+        rows, cols, amounts = [], [], []
+        for i, seq in enumerate(seqs):
+            if seq.params.presence_penalty != 0:
+                seen = set(seq.output_ids)
+                rows.extend([i] * len(seen))
+                cols.extend(seen)
+                amounts.extend([seq.params.presence_penalty] * len(seen))
+        if not rows:
+            return logits
+        logits = logits.clone()
+        ops.apply_penalty(
+            logits,
+            torch.tensor(rows, dtype=torch.int32).to(self.device),
+            torch.tensor(cols, dtype=torch.int32).to(self.device),
+            torch.tensor(amounts, dtype=torch.float32).to(self.device),
+        )
+        return logits
+
+
+def _as_int64(seed: int) -> int:
+    seed &= (1 << 64) - 1
+    return seed - (1 << 64) if seed >= (1 << 63) else seed

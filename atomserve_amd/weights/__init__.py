@@ -1,0 +1,4 @@
+from atomserve_amd.weights.loader import WeightsError, bind_checkpoint, load_model, load_weights
+from atomserve_amd.weights.random_init import random_checkpoint, write_random_model
+
+__all__ = ["WeightsError", "bind_checkpoint", "load_model", "load_weights", "random_checkpoint", "write_random_model"]
