@@ -17,6 +17,11 @@
 
 #define NEG_INF (-__builtin_inff())
 
+// exp of the fp32 path is the precise one; bf16 serving uses the hardware approximation.
+template <typename T> __device__ __forceinline__ float fexp(float x);
+template <> __device__ __forceinline__ float fexp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ float fexp<bf16>(float x) { return __expf(x); }
+
 template <typename T> struct Chunk;  // 16 bytes of a head
 template <> struct Chunk<float> {
   static constexpr int N = 4;
@@ -123,8 +128,8 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
 #pragma unroll
       for (int g = 0; g < GT; ++g) {
         const float mn = fmaxf(m[g], s[g]);
-        const float a = __expf(m[g] - mn);  // m = -inf gives 0
-        const float p = __expf(s[g] - mn);
+        const float a = fexp<T>(m[g] - mn);  // m = -inf gives 0
+        const float p = fexp<T>(s[g] - mn);
         l[g] = l[g] * a + p;
 #pragma unroll
         for (int c = 0; c < CH; ++c) acc[g][c] = acc[g][c] * a + p * vv[c];
@@ -139,8 +144,8 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
     for (int g = 0; g < GT; ++g) {
       const float mo = __shfl_xor(m[g], off, WAVE), lo_ = __shfl_xor(l[g], off, WAVE);
       const float mn = fmaxf(m[g], mo);
-      const float a = (m[g] == NEG_INF) ? 0.f : __expf(m[g] - mn);
-      const float b = (mo == NEG_INF) ? 0.f : __expf(mo - mn);
+      const float a = (m[g] == NEG_INF) ? 0.f : fexp<T>(m[g] - mn);
+      const float b = (mo == NEG_INF) ? 0.f : fexp<T>(mo - mn);
       l[g] = l[g] * a + lo_ * b;
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       const float mw = sm[w * GT + g];
-      const float e = (mw == NEG_INF) ? 0.f : __expf(mw - mx);
+      const float e = (mw == NEG_INF) ? 0.f : fexp<T>(mw - mx);
       num += sacc[((size_t)w * GT + g) * D + d] * e;
       den += sl[w * GT + g] * e;
     }
@@ -202,14 +207,14 @@ __global__ void attn_reduce_kernel(const int* __restrict__ items, const float* _
   float den = 0.f;
   for (int p = 0; p < P; ++p) {
     const float mp = part_m[o + p];
-    den += (mp == NEG_INF) ? 0.f : part_l[o + p] * __expf(mp - mx);
+    den += (mp == NEG_INF) ? 0.f : part_l[o + p] * fexp<T>(mp - mx);
   }
   const int t = items[item];
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float num = 0.f;
     for (int p = 0; p < P; ++p) {
       const float mp = part_m[o + p];
-      if (mp != NEG_INF) num += part_acc[(o + p) * D + d] * __expf(mp - mx);
+      if (mp != NEG_INF) num += part_acc[(o + p) * D + d] * fexp<T>(mp - mx);
     }
     out[((size_t)t * H + h) * D + d] = from_f32<T>(num / den);
   }

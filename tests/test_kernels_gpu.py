@@ -1,0 +1,385 @@
+"""Each HIP kernel alone against its plain reference (tests/plain_kernels.py), at sizes
+other than the tiny models'.  fp32 differences are real faults; bf16 results may differ
+from the rounded reference by one rounding step."""
+
+import math
+
+import pytest
+import torch
+
+from tests import plain_kernels as pk
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from atomserve_amd.kernels import ops as module
+
+    return module
+
+
+def close_bf16(got, ref, scale=None):
+    """Equal to the reference rounded to bfloat16, up to one step of the larger magnitude."""
+    got, ref = got.float(), ref.float()
+    step = torch.maximum(ref.abs(), got.abs()) * 2.0**-7 + (1e-6 if scale is None else scale * 2.0**-8)
+    return bool(((got - ref).abs() <= step).all())
+
+
+def i32(values):
+    return torch.tensor(values, dtype=I32, device=DEV)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embed_gather(ops, dtype):
+    torch.manual_seed(0)
+    table = torch.randn(1000, 96, device=DEV).to(dtype)
+    ids = i32([0, 999, 5, 5, 731, 12, 1])
+    out = torch.full((7, 96), 7.0, device=DEV)
+    ops.embed_gather(table, ids, out)
+    assert torch.equal(out, pk.embed_gather(table, ids))
+
+
+@pytest.mark.parametrize("n", [96, 1000, 4096, 5120])
+@pytest.mark.parametrize("rows", [1, 7, 300])
+def test_rmsnorm_fp32(ops, n, rows):
+    torch.manual_seed(1)
+    x = torch.randn(rows, n, device=DEV) * 3
+    w = torch.randn(n, device=DEV) + 1
+    out = torch.empty_like(x)
+    ops.rmsnorm(x, w, 1e-5, out)
+    ref, _ = pk.rmsnorm(x, w, 1e-5)
+    assert torch.allclose(out, ref, atol=1e-5, rtol=1e-6)
+
+
+@pytest.mark.parametrize("out_dtype,w_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
+def test_rmsnorm_adds_the_pending_delta_and_selects_rows(ops, out_dtype, w_dtype):
+    torch.manual_seed(2)
+    T, n = 37, 200
+    x0 = torch.randn(T, n, device=DEV) * 2
+    delta = torch.randn(T, n, device=DEV).to(out_dtype)
+    w = (torch.randn(n, device=DEV) * 0.2 + 1).to(w_dtype)
+    # fused sum, written back
+    x = x0.clone()
+    out = torch.empty(T, n, dtype=out_dtype, device=DEV)
+    ops.rmsnorm(x, w, 1e-6, out, delta=delta)
+    ref, new_x = pk.rmsnorm(x0, w, 1e-6, delta)
+    assert torch.allclose(x, new_x, atol=1e-6)
+    assert torch.allclose(out.float(), ref, atol=1e-5) if out_dtype == F32 else close_bf16(out, ref)
+    # row selection without touching x
+    rows = i32([36, 0, 5, 5])
+    x = x0.clone()
+    out = torch.empty(4, n, dtype=out_dtype, device=DEV)
+    ops.rmsnorm(x, w, 1e-6, out, delta=delta, rows=rows, update_x=False)
+    ref, _ = pk.rmsnorm(x0, w, 1e-6, delta, rows)
+    assert torch.equal(x, x0)
+    assert torch.allclose(out.float(), ref, atol=1e-5) if out_dtype == F32 else close_bf16(out, ref)
+
+
+def test_rmsnorm_eps_matters(ops):
+    x = torch.full((1, 64), 1e-3, device=DEV)
+    w = torch.ones(64, device=DEV)
+    a, b = torch.empty_like(x), torch.empty_like(x)
+    ops.rmsnorm(x, w, 1e-6, a)
+    ops.rmsnorm(x, w, 1e-2, b)
+    assert torch.allclose(a, torch.full_like(a, 1e-3 / math.sqrt(2e-6)), rtol=1e-5)
+    assert torch.allclose(b, torch.full_like(b, 1e-3 / math.sqrt(1e-6 + 1e-2)), rtol=1e-5)
+
+
+def test_rope_table_large_positions(ops):
+    # positions from reference tests/test_kernels.py:35, theta 1e6
+    pos = i32([0, 1, 300, 4097, 39999])
+    inv = (1.0 / (1e6 ** (torch.arange(0, 128, 2, dtype=torch.float64) / 128))).to(DEV)
+    out = torch.empty(5, 64, 2, device=DEV)
+    ops.rope_table(pos, inv, out)
+    assert torch.allclose(out, pk.rope_table(pos, inv), atol=2e-7, rtol=0)
+    assert torch.equal(out[0, :, 0], torch.ones(64, device=DEV)) and torch.equal(out[0, :, 1], torch.zeros(64, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("heads,D,bs", [((16, 8), 128, 16), ((32, 8), 128, 16), ((6, 2), 32, 8), ((5, 5), 48, 4), ((4, 1), 16, 16)])
+def test_qk_norm_rope_store(ops, dtype, heads, D, bs):
+    H, KV = heads
+    torch.manual_seed(3)
+    pos = i32([0, 1, 300, 4097, 39999])
+    slots = i32([3, 9, 17, 2, 30])
+    qkv = (torch.randn(5, H + 2 * KV, D, device=DEV) * 3).to(dtype)
+    qw, kw = (torch.randn(D, device=DEV) + 1).to(dtype), (torch.randn(D, device=DEV) + 1).to(dtype)
+    inv = (1.0 / (1e6 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))).to(DEV)
+    cs = torch.empty(5, D // 2, 2, device=DEV)
+    ops.rope_table(pos, inv, cs)
+    pages = 64 // bs
+    k_pages = torch.zeros(pages, KV, bs, D, dtype=dtype, device=DEV)
+    v_pages = torch.zeros_like(k_pages)
+    q = torch.empty(5, H, D, dtype=dtype, device=DEV)
+    ops.qk_norm_rope_store(qkv, qw, kw, cs, slots, q, k_pages, v_pages, H, KV, 1e-6)
+    rq, rk, rv = pk.qk_norm_rope(qkv, qw, kw, cs, H, KV, 1e-6)
+    ref_k, ref_v = torch.zeros(pages, KV, bs, D, device=DEV), torch.zeros(pages, KV, bs, D, device=DEV)
+    pk.store_pages(ref_k, ref_v, rk, rv, slots)
+    if dtype == F32:
+        assert torch.allclose(q, rq, atol=1e-5) and torch.allclose(k_pages, ref_k, atol=1e-5)
+    else:
+        assert close_bf16(q, rq) and close_bf16(k_pages, ref_k)
+    assert torch.equal(v_pages.float(), ref_v)  # values are copied bit for bit; untouched slots stay zero
+    assert (k_pages.float().abs().sum(dim=(1, 3)) > 0).sum() == 5
+
+
+def test_qk_norm_rope_store_variants(ops):
+    """No norm, no rotation, a rotation of part of the head, and q alone (a run that reads
+    another run's cache stores nothing)."""
+    torch.manual_seed(4)
+    H, KV, D = 4, 2, 32
+    qkv = torch.randn(3, H + 2 * KV, D, device=DEV)
+    pos, slots = i32([5, 6, 7]), i32([0, -1, 9])
+    inv = (1.0 / (1e4 ** (torch.arange(0, 16, 2, dtype=torch.float64) / 16))).to(DEV)
+    cs = torch.empty(3, 8, 2, device=DEV)
+    ops.rope_table(pos, inv, cs)
+    k_pages, v_pages = torch.zeros(2, KV, 8, D, device=DEV), torch.zeros(2, KV, 8, D, device=DEV)
+    q = torch.empty(3, H, D, device=DEV)
+    ops.qk_norm_rope_store(qkv, None, None, cs, slots, q, k_pages, v_pages, H, KV, 0.0)
+    rq, rk, rv = pk.qk_norm_rope(qkv, None, None, cs, H, KV, 0.0)
+    assert torch.allclose(q, rq, atol=1e-6)
+    assert torch.equal(q[..., 16:], qkv[:, :H, 16:])  # beyond the rotary width nothing changes
+    assert torch.allclose(k_pages[0, :, 0], rk[0], atol=1e-6) and torch.allclose(k_pages[1, :, 1], rk[2], atol=1e-6)
+    assert k_pages.abs().sum(dim=(1, 3)).count_nonzero() == 2  # the token with slot -1 stored nothing
+    q2 = torch.empty_like(q)
+    ops.qk_norm_rope_store(qkv, None, None, None, None, q2, None, None, H, KV, 0.0, store_kv=False)
+    assert torch.equal(q2, qkv[:, :H])
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("rows,inter", [(1, 3072), (7, 3072), (300, 3072), (5, 160)])
+def test_silu_mul(ops, dtype, rows, inter):
+    # sizes from reference tests/test_kernels.py:192-198
+    torch.manual_seed(5)
+    gu = (torch.randn(rows, 2 * inter, device=DEV) * 3).to(dtype)
+    out = torch.empty(rows, inter, dtype=dtype, device=DEV)
+    ops.silu_mul(gu, out)
+    ref = pk.silu_mul(gu)
+    assert torch.allclose(out, ref, atol=1e-5) if dtype == F32 else close_bf16(out, ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 1000, 96), (130, 257, 193), (64, 64, 16), (65, 63, 17), (3, 2000, 4096)])
+def test_gemm_fp32_is_true_fp32(ops, M, N, K):
+    torch.manual_seed(6)
+    a, w = torch.randn(M, K, device=DEV), torch.randn(N, K, device=DEV)
+    out = torch.empty(M, N, device=DEV)
+    ops.gemm(a, w, out)
+    ref = pk.gemm(a, w)
+    assert torch.allclose(out, ref, atol=2e-6 * math.sqrt(K) * 4, rtol=1e-6)
+    # a reduced-precision matrix mode (bf16 or tf32-like inputs) would be off by about 1e-3 * sqrt(K)
+    assert (out - ref).abs().max() < 1e-4 * math.sqrt(K)
+
+
+def test_gemm_fp32_rows_do_not_depend_on_the_batch(ops):
+    torch.manual_seed(7)
+    a, w = torch.randn(70, 200, device=DEV), torch.randn(300, 200, device=DEV)
+    full = torch.empty(70, 300, device=DEV)
+    ops.gemm(a, w, full)
+    for i in (0, 63, 64, 69):
+        one = torch.empty(1, 300, device=DEV)
+        ops.gemm(a[i : i + 1].contiguous(), w, one)
+        assert torch.equal(one[0], full[i])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (64, 4096, 1024), (300, 257, 192), (5, 2000, 4096)])
+def test_gemm_bf16(ops, M, N, K):
+    torch.manual_seed(8)
+    a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
+    ref = pk.gemm(a, w)
+    out = torch.empty(M, N, dtype=BF16, device=DEV)
+    ops.gemm(a, w, out)
+    assert close_bf16(out, ref, scale=math.sqrt(K))
+    out32 = torch.empty(M, N, dtype=F32, device=DEV)
+    ops.gemm(a, w, out32)
+    assert torch.allclose(out32, ref, atol=math.sqrt(K) * 2.0**-8, rtol=2.0**-7)
+
+
+def paged_case(dtype, H, KV, D, bs, lens, seed=0, k_scale=4.0):
+    """Random pools and scattered block tables for contexts of the given lengths; the query of
+    request i sits at position lens[i] - 1."""
+    g = torch.Generator().manual_seed(seed)
+    pages = sum(-(-n // bs) for n in lens) + 8
+    k_pages = (torch.randn(pages, KV, bs, D, generator=g) * k_scale).to(dtype).to(DEV)
+    v_pages = torch.randn(pages, KV, bs, D, generator=g).to(dtype).to(DEV)
+    perm = torch.randperm(pages, generator=g).tolist()
+    tables, at = [], 0
+    for n in lens:
+        nb = -(-n // bs)
+        tables.append(perm[at : at + nb])
+        at += nb
+    width = max(map(len, tables))
+    padded = i32([t + [0] * (width - len(t)) for t in tables])
+    q = torch.randn(len(lens), H, D, generator=g).to(dtype).to(DEV)
+    positions = i32([n - 1 for n in lens])
+    return q, k_pages, v_pages, padded, positions
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("H,KV,D,bs", [(16, 8, 128, 16), (32, 8, 128, 16), (8, 8, 128, 16), (6, 2, 32, 8),
+                                       (4, 2, 16, 16), (5, 1, 48, 4), (16, 1, 64, 32), (64, 8, 128, 16)])  # fmt: skip
+def test_attention_single_query(ops, dtype, H, KV, D, bs):
+    """Contexts of one key, part of a page, exactly one partition and several partitions, on
+    scattered pages (lengths from reference tests/test_kernels.py:98-125)."""
+    if dtype == BF16 and D % 8:
+        pytest.skip("bf16 heads come in steps of 8")
+    lens = [1, 37, 512, 513, 1500]
+    q, k_pages, v_pages, tables, positions = paged_case(dtype, H, KV, D, bs, lens, k_scale=4.0 / math.sqrt(D / 16))
+    rows = i32(list(range(len(lens))))
+    items = i32(list(range(len(lens))))
+    out = torch.zeros(len(lens), H, D, dtype=dtype, device=DEV)
+    scale = D**-0.5
+    ref = pk.paged_attention(q, k_pages, v_pages, items, positions, rows, tables, scale)
+    for part_size in (None, 256, 64):
+        out.zero_()
+        ops.attn_single_query(q, k_pages, v_pages, items, positions, rows, tables, out, scale, 0, max(lens), part_size)
+        if dtype == F32:
+            assert torch.allclose(out, ref, atol=1e-5), f"partitions of {part_size}: {(out - ref).abs().max()}"
+        else:
+            assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), f"{(out.float() - ref).abs().max()}"
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_finds_one_far_key_among_many(ops, dtype):
+    """One key far back matches the query strongly; the result must be (almost) that key's value,
+    wherever in the context, the pages and the partitions it lies."""
+    H, KV, D, bs, n = 8, 2, 64, 16, 1500
+    for far in (0, 15, 16, 255, 256, 700, 1498, 1499):
+        q, k_pages, v_pages, tables, positions = paged_case(dtype, H, KV, D, bs, [n], seed=far, k_scale=0.05)
+        page, off = int(tables[0, far // bs]), far % bs
+        G = H // KV
+        for kvh in range(KV):  # the first query head of each group gets its match
+            k_pages[page, kvh, off] = (q[0, kvh * G].float() * 4.0).to(dtype)
+        out = torch.zeros(1, H, D, dtype=dtype, device=DEV)
+        ops.attn_single_query(q, k_pages, v_pages, i32([0]), positions, i32([0]), tables, out, 1.0, 0, n)
+        for kvh in range(KV):
+            want = v_pages[page, kvh, off].float()
+            assert torch.allclose(out[0, kvh * G].float(), want, atol=2e-2), (far, kvh)
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 300])
+def test_attention_window_edge(ops, window):
+    H, KV, D, bs = 4, 2, 32, 8
+    lens = [1, 9, 100, 513]
+    q, k_pages, v_pages, tables, positions = paged_case(F32, H, KV, D, bs, lens)
+    items = rows = i32(list(range(4)))
+    out = torch.zeros(4, H, D, device=DEV)
+    ops.attn_single_query(q, k_pages, v_pages, items, positions, rows, tables, out, D**-0.5, window, max(lens), 64)
+    ref = pk.paged_attention(q, k_pages, v_pages, items, positions, rows, tables, D**-0.5, window)
+    assert torch.allclose(out, ref, atol=1e-5)
+
+
+def test_attention_serves_only_the_listed_tokens(ops):
+    """Items select tokens; several tokens of one request share a table and see keys up to
+    their own position only."""
+    H, KV, D, bs = 4, 2, 32, 8
+    q, k_pages, v_pages, tables, _ = paged_case(F32, H, KV, D, bs, [40])
+    q = torch.randn(6, H, D, device=DEV)
+    positions, rows = i32([3, 4, 5, 37, 38, 39]), i32([0] * 6)
+    items = i32([1, 4, 5])
+    out = torch.full((6, H, D), 9.0, device=DEV)
+    ops.attn_single_query(q, k_pages, v_pages, items, positions, rows, tables, out, D**-0.5, 0, 40)
+    ref = pk.paged_attention(q, k_pages, v_pages, items, positions, rows, tables, D**-0.5)
+    assert torch.allclose(out[[1, 4, 5]], ref[[1, 4, 5]], atol=1e-5)
+    assert bool((out[[0, 2, 3]] == 9.0).all())
+
+
+def test_kernels_refuse_what_they_cannot_do(ops):
+    from atomserve_amd.kernels.lib import KernelError
+
+    x = torch.zeros(2, 8, device=DEV)
+    with pytest.raises(KernelError):
+        ops.rmsnorm(x, torch.ones(9, device=DEV), 1e-6, torch.empty_like(x))
+    with pytest.raises(KernelError):
+        ops.rmsnorm(x.cpu(), torch.ones(8), 1e-6, torch.empty(2, 8))
+    q = torch.zeros(1, 2, 6, device=DEV)
+    with pytest.raises(KernelError, match="head width"):
+        ops.attn_single_query(q, torch.zeros(1, 1, 4, 6, device=DEV), torch.zeros(1, 1, 4, 6, device=DEV), i32([0]),
+                              i32([0]), i32([0]), i32([[0]]), torch.zeros_like(q), 1.0, 0, 1)  # fmt: skip
+
+
+# ---- sampling -------------------------------------------------------------------------
+
+
+def test_argmax_and_ties(ops):
+    torch.manual_seed(9)
+    logits = torch.randn(7, 151936, device=DEV) * 4
+    out = torch.empty(7, dtype=I32, device=DEV)
+    ops.argmax(logits, out)
+    assert out.tolist() == logits.argmax(dim=-1).tolist()
+    ties = torch.zeros(2, 1000, device=DEV)
+    ties[0, [17, 400]] = 3.0
+    ties[1, :] = float("-inf")
+    ties[1, 999] = -5.0
+    out = torch.empty(2, dtype=I32, device=DEV)
+    ops.argmax(ties, out)
+    assert out.tolist() == [17, 999]
+
+
+def test_topk_matches_the_library(ops):
+    """Exact values for every k, with heavy ties and rows with fewer finite entries than k
+    (cases of reference tests/test_kernels.py:155-171)."""
+    torch.manual_seed(10)
+    cases = [
+        torch.randn(7, 151936, device=DEV) * 4,
+        torch.randint(-5, 5, (3, 151936), device=DEV).float(),
+        torch.full((2, 151936), float("-inf"), device=DEV).index_fill_(1, torch.tensor([3, 9], device=DEV), 1.0),
+    ]
+    for x in cases:
+        for k in (1, 2, 20, 33, 64):
+            values = torch.empty(x.shape[0], k, device=DEV)
+            indices = torch.empty(x.shape[0], k, dtype=I32, device=DEV)
+            ops.topk(x, k, values, indices)
+            expected = pk.topk_values(x, k)
+            assert torch.equal(values, expected)
+            assert torch.equal(x.gather(1, indices.long().clamp_min(0)), expected)
+
+
+def sample_rows(ops, logits, temperature, top_k, top_p, seeds, counters=None):
+    B = logits.shape[0]
+    out = torch.empty(B, dtype=I32, device=DEV)
+    f = lambda v: torch.full((B,), v, dtype=F32, device=DEV) if not torch.is_tensor(v) else v  # noqa: E731
+    ops.sample(logits, f(temperature), torch.full((B,), top_k, dtype=I32, device=DEV) if not torch.is_tensor(top_k) else top_k,
+               f(top_p), torch.as_tensor(seeds, dtype=torch.int64).to(DEV),
+               torch.zeros(B, dtype=I32, device=DEV) if counters is None else counters, out)  # fmt: skip
+    return out
+
+
+PROBS = torch.tensor([0.4, 0.3, 0.2, 0.1])
+
+
+def test_sampling_follows_the_distribution(ops):
+    """Frequencies over 20,000 draws (reference tests/test_sampler.py:33-47), through the
+    top-k path and through the all-tokens path."""
+    n = 20000
+    logits = PROBS.log().repeat(n, 1).to(DEV)
+    seeds = torch.arange(n) * 7919 + 1
+    for top_k in (0, 3):
+        draws = sample_rows(ops, logits, 1.0, top_k, 1.0, seeds)
+        freq = draws.long().bincount(minlength=4).float().cpu() / n
+        want = PROBS if top_k == 0 else torch.tensor([0.4, 0.3, 0.2, 0.0]) / 0.9
+        assert torch.allclose(freq, want, atol=0.015), (top_k, freq)
+    assert set(sample_rows(ops, logits[:2000], 1.0, 2, 1.0, seeds[:2000]).tolist()) == {0, 1}
+    assert set(sample_rows(ops, logits[:200], 1.0, 1, 1.0, seeds[:200]).tolist()) == {0}
+    for top_k in (0, 4):  # top-p through both paths
+        assert set(sample_rows(ops, logits[:2000], 1.0, top_k, 0.6, seeds[:2000]).tolist()) == {0, 1}
+        assert set(sample_rows(ops, logits[:200], 1.0, top_k, 0.01, seeds[:200]).tolist()) == {0}
+    sharp = sample_rows(ops, logits, 0.5, 0, 1.0, seeds).long().bincount(minlength=4).float().cpu() / n
+    assert torch.allclose(sharp, PROBS**2 / (PROBS**2).sum(), atol=0.015)
+
+
+def test_sampling_is_seeded_per_request_and_mixes_greedy_rows(ops):
+    torch.manual_seed(11)
+    row = torch.randn(1, 1000, device=DEV)
+    alone = [int(sample_rows(ops, row, 1.0, 50, 1.0, [7], i32([c]))[0]) for c in range(20)]
+    crowd = []
+    for c in range(20):
+        logits = torch.cat([torch.randn(1, 1000, device=DEV), row, torch.randn(1, 1000, device=DEV)])
+        t = torch.tensor([0.8, 1.0, 0.0], device=DEV)
+        k = i32([500, 50, 20])
+        out = sample_rows(ops, logits, t, k, torch.tensor([0.9, 1.0, 0.95], device=DEV), [3, 7, 5], i32([c, c, c]))
+        crowd.append(int(out[1]))
+        assert int(out[2]) == int(logits[2].argmax())  # the greedy row is its argmax
+    assert alone == crowd and len(set(alone)) > 1

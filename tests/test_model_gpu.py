@@ -1,0 +1,145 @@
+"""The engine against the plain implementation on a real GPU, in 32-bit and in bfloat16:
+the same requests whole, decoded one by one, in portions, and mixed with few pages."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import plain_qwen3 as plain
+from tests import replay_cases as rc
+from tests.conftest import ROOT, TINY, plain_random_weights, write_model_dir
+
+pytestmark = pytest.mark.gpu
+
+# fp32: the engine and the float64 plain implementation differ by fp32 rounding only.
+# bf16: activations carry 8 bits; the bound is a few rounding steps of the largest logit.
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+LENGTHS = {"A": 200, "B": 420}
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def setup(request, tmp_path_factory):
+    name = request.param
+    raw = TINY[name]
+    weights = plain_random_weights(raw, seed=41 if name == "A" else 43, std=0.2, gain_std=0.2)
+    path = write_model_dir(str(tmp_path_factory.mktemp(f"tiny{name}")), raw, weights, torch.bfloat16)
+    return name, raw, weights, path, {}
+
+
+def make_replay(path, dtype, max_tokens):
+    from atomserve_amd.engine.replay import Replay
+
+    return Replay(path, dtype, max_tokens)
+
+
+def check(worst, scale, dtype):
+    assert worst <= TOL[dtype] * max(scale, 1.0), f"{dtype}: |difference| {worst:.3e} against |logits| {scale:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_decoded_and_in_portions(setup, dtype):
+    name, raw, weights, path, cache = setup
+    ids = rc.random_ids(raw["vocab_size"], LENGTHS[name], seed=1)
+    requests = {"a": ids}
+    for steps in (rc.whole("a", ids), rc.prefill_then_decode("a", ids), rc.portions("a", ids)):
+        replay = make_replay(path, dtype, rc.live_token_bound(steps))
+        worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
+        assert rows >= 33
+        check(worst, scale, dtype)
+        assert replay.manager.num_free == replay.manager.num_blocks  # everything was given back
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_requests_with_pages_used_again(setup, dtype):
+    name, raw, weights, path, cache = setup
+    lengths = [70, 33, 150, 64, 97, 20, 129, 65] if name == "A" else [90, 300, 64, 17, 257, 128, 40, 200]
+    requests = {f"r{i}": rc.random_ids(raw["vocab_size"], n, seed=100 + i) for i, n in enumerate(lengths)}
+    steps = rc.mixed(requests, seed=5)
+    bound = rc.live_token_bound(steps)
+    assert bound < sum(-(-n // 64) * 64 for n in lengths)  # fewer pages than all requests need: reuse
+    replay = make_replay(path, dtype, bound)
+    worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
+    assert rows > 200
+    check(worst, scale, dtype)
+    assert replay.manager.num_free == replay.manager.num_blocks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_long_decoding(setup, dtype):
+    name, raw, weights, path, cache = setup
+    n = LENGTHS[name]
+    ids = rc.random_ids(raw["vocab_size"], n, seed=2)
+    steps = [{"step": i, "entries": [{"id": "d", "tokens": [ids[i]], "want": [0]}], "end": []} for i in range(n)]
+    replay = make_replay(path, dtype, n + 64)
+    worst, scale, rows = rc.run_and_compare(replay, steps, {"d": ids}, raw, weights, cache)
+    assert rows == n
+    check(worst, scale, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(setup, dtype, tmp_path):
+    """The program itself, as a user starts it: JSON lines in, <step>.f32 files and `done` lines out."""
+    name, raw, weights, path, cache = setup
+    ids = rc.random_ids(raw["vocab_size"], 50, seed=3)
+    other = rc.random_ids(raw["vocab_size"], 21, seed=4)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": ids[:30], "want": [0, 29]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": ids[30:33], "want": []}, {"id": "b", "tokens": other, "want": [20]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": ids[33:], "want": [16]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", path, "--dtype", dtype, "--out", str(out),
+         "--max-tokens", "128"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
+    )  # fmt: skip
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2"]
+    ref_a, ref_b = plain.logits(raw, weights, ids).float().numpy(), plain.logits(raw, weights, other).float().numpy()
+    got0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1)
+    got1 = np.fromfile(out / "1.f32", dtype="<f4").reshape(1, -1)
+    got2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1)
+    for got, want in ((got0[0], ref_a[0]), (got0[1], ref_a[29]), (got1[0], ref_b[20]), (got2[0], ref_a[49])):
+        assert np.abs(got - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_greedy_generation_through_the_entry_point(setup, dtype):
+    """Greedy tokens through engine, scheduler, cache and kernels equal recomputing the whole
+    sequence for every token; batched, chunked and preempted runs give the same tokens (fp32)."""
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.weights import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, dtype, "cuda:0")
+    prompts = [rc.random_ids(raw["vocab_size"], n, seed=200 + n) for n in (5, 17, 33, 1)]
+    params = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
+    bs = 16 if name == "A" else 8
+
+    def engine(**kw):
+        cfg = {"block_size": bs, "num_blocks": 64, "max_model_len": 128, "max_num_seqs": 8, **kw}
+        return create_engine(model, EngineConfig(**cfg))
+
+    together = engine().generate(prompts, params)
+    if dtype == torch.float32:
+        assert together == [plain.greedy(raw, weights, p, 20) for p in prompts]
+        assert engine(max_num_batched_tokens=8, max_num_seqs=4).generate(prompts, params) == together
+        # exactly the pages the prompts need: every request that grows evicts a newer one
+        tight = engine(num_blocks=sum(-(-len(p) // bs) for p in prompts), max_model_len=64)
+        assert tight.generate(prompts, params) == together
+        assert tight.stats()["preemptions"] > 0 and tight.stats()["kv_blocks_used"] == 0
+    else:
+        # bf16 may flip near-ties; every token must still be (nearly) the best under the plain logits
+        for p, out in zip(prompts, together):
+            seq = list(p)
+            for t in out:
+                ref = plain.logits(raw, weights, seq)[-1]
+                assert ref[t] >= ref.max() - TOL["bfloat16"] * max(1.0, float(ref.abs().max())) * 2
+                seq.append(t)
