@@ -1,0 +1,172 @@
+"""Decode and prefill throughput of random-weight Qwen3-8B layer sizes on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
+Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
+plus prefill of 2,048 tokens, the decode roofline and the batch 1 and 64 points.
+Method as in the reference's bench/engine.py: synthetic token ids, prefix caching off,
+ignore_eos, warm-up first, prompt steps outside the decode timer, tokens counted.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}  # dense MFMA
+
+# Qwen3-8B layer sizes (BASELINE.json configs[2])
+SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_layers=36, num_heads=32,
+             num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
+             max_position_embeddings=40960)  # fmt: skip
+FULL_LAYERS = 36
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=128)
+    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--context", type=int, default=2048)
+    p.add_argument("--layers", type=int, default=FULL_LAYERS)
+    p.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    p.add_argument("--points", default="1,64", help="other decode batch sizes to measure (fewer steps each)")
+    p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--greedy", action="store_true", help="greedy instead of the default sampling settings")
+    return p.parse_args()
+
+
+def prompt(b: int, n: int, vocab: int) -> list:
+    """Distinct synthetic prompts (reference bench/engine.py:90-92)."""
+    return [(1000 + 37 * b + i) % (vocab - 1000) for i in range(n)]
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
+        return 2
+
+    import torch
+
+    from atomserve_amd.config import EngineConfig, Qwen3Config
+    from atomserve_amd.config.registry import architecture_for
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.models.decoder import DecoderModel
+    from atomserve_amd.weights.loader import DictSource, bind_checkpoint
+    from atomserve_amd.weights.random_init import random_checkpoint
+
+    device = "cuda:0"
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    config = Qwen3Config(**{**SIZES, "num_layers": args.layers})
+    arch = architecture_for(config.to_dict())
+    model = DecoderModel(arch.build_plan(config), dtype, device)
+    bind_checkpoint(model, arch, config, DictSource(random_checkpoint(arch, config, seed=0, dtype=dtype, device=device)))
+    torch.cuda.synchronize()
+
+    batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
+    block = 16
+    max_len = 4096
+    num_blocks = max(batches) * max_len // block
+    params = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True) if args.greedy else \
+        SamplingParams(max_tokens=100000, ignore_eos=True)  # fmt: skip
+    engine_config = EngineConfig(block_size=block, num_blocks=num_blocks, max_num_seqs=max(batches),
+                                 max_num_batched_tokens=max(2048, args.context), max_model_len=max_len,
+                                 enable_prefix_caching=False)  # fmt: skip
+    engine = create_engine(model, engine_config, seed=0)
+
+    itemsize = 2 if args.dtype == "bf16" else 4
+    c = config
+    layer_params = c.hidden_size * (c.num_heads + 2 * c.num_kv_heads) * c.head_dim + c.num_heads * c.head_dim * c.hidden_size \
+        + 3 * c.hidden_size * c.intermediate_size  # fmt: skip
+    weight_bytes = (layer_params * c.num_layers + c.vocab_size * c.hidden_size) * itemsize
+    kv_bytes_per_token = c.num_layers * 2 * c.num_kv_heads * c.head_dim * itemsize
+
+    def run_decode(batch: int, steps: int, warmup: int):
+        """Prefill `batch` prompts of args.context tokens (untimed), then time `steps` decode steps."""
+        handles = [engine.submit(prompt(b, args.context, c.vocab_size), params) for b in range(batch)]
+        while any(s.num_computed_tokens < s.num_prompt_tokens for s in
+                  [*engine.scheduler.running, *engine.scheduler.waiting]) or engine.scheduler.waiting or not engine.scheduler.running:
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        ctx_start = engine.scheduler.running[0].num_tokens
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert len(engine.scheduler.running) == batch and engine.last_batch_tokens == batch
+        mean_ctx = ctx_start + steps / 2
+        for h in handles:
+            engine.abort(h.id)
+        engine.step()
+        assert engine.stats()["kv_blocks_used"] == 0
+        return batch * steps / dt, dt / steps * 1e3, mean_ctx
+
+    result_prefill = None
+    if not args.no_prefill:
+        one = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+        engine.generate([prompt(99, 2048, c.vocab_size)], one)  # warm-up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.generate([prompt(98, 2048, c.vocab_size)], one)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        T = 2048
+        flops = 2 * T * layer_params * c.num_layers + 2 * c.hidden_size * c.vocab_size \
+            + 4 * c.num_heads * c.head_dim * (T * (T + 1) // 2) * c.num_layers  # fmt: skip
+        result_prefill = {"value": round(T / dt, 1), "tokens": T, "ms": round(dt * 1e3, 3),
+                          "frac": round(flops / dt / PEAK_FLOPS[args.dtype], 4)}  # fmt: skip
+
+    points = {}
+    for b in batches:
+        if b != args.batch:
+            tps, ms, _ = run_decode(b, max(16, args.steps // 4), max(2, args.warmup // 2))
+            points[f"decode_b{b}"] = round(tps, 1)
+    tps, ms, mean_ctx = run_decode(args.batch, args.steps, args.warmup)
+    step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
+    achieved = step_bytes / (ms * 1e-3)
+
+    line = {
+        "metric": "decode tok/s at batch 8, 2048-token contexts (Qwen3-8B sizes, random weights)",
+        "value": round(tps, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic token ids, random-init weights",
+        "config": {
+            "model": "Qwen3-8B sizes", "layers": c.num_layers, "layers_full": FULL_LAYERS, "hidden": c.hidden_size,
+            "heads": c.num_heads, "kv_heads": c.num_kv_heads, "head_dim": c.head_dim,
+            "intermediate": c.intermediate_size, "vocab": c.vocab_size, "global_batch": args.batch,
+            "seq_len": args.context, "max_context": max_len, "block_size": block, "parallelism": "single GPU",
+            "sampling": "greedy" if args.greedy else "temperature 0.6 top-k 20 top-p 0.95",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},  # fmt: skip
+        "points": points,
+    }
+    if result_prefill:
+        line["prefill"] = result_prefill
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
