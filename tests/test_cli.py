@@ -1,0 +1,52 @@
+"""The command-line surface (argument parsing only; no model is loaded;
+reference tests/test_cli.py:9-51)."""
+
+import pytest
+
+from atomserve_amd import __version__
+from atomserve_amd.engine.cli import build_parser, engine_config_for, main, parse_ids
+
+
+def test_help_version_and_required_model(capsys):
+    with pytest.raises(SystemExit) as exc:
+        main(["--help"])
+    assert exc.value.code == 0 and "usage: atomserve" in capsys.readouterr().out
+    with pytest.raises(SystemExit) as exc:
+        main(["--version"])
+    assert exc.value.code == 0 and __version__ in capsys.readouterr().out
+    with pytest.raises(SystemExit) as exc:
+        build_parser().parse_args([])
+    assert exc.value.code == 2
+    assert build_parser().parse_args(["Qwen/Qwen3-0.6B"]).model == "Qwen/Qwen3-0.6B"
+
+
+def test_reference_option_names_and_defaults():
+    a = build_parser().parse_args(["m"])
+    assert (a.dtype, a.kv_mem_gb, a.block_size, a.max_num_seqs, a.max_batched_tokens, a.no_prefix_caching) == (
+        "bf16", 4.0, 16, 32, 512, False)  # fmt: skip
+    assert (a.temperature, a.top_k, a.top_p) == (0.6, 20, 0.95)
+
+
+def test_pool_is_sized_from_the_memory_budget():
+    """4 GiB of bf16 cache at 1.75 MiB per 16-token block of Qwen3-0.6B is 2340 blocks."""
+    block_bytes = 28 * 2 * 8 * 128 * 2 * 16
+    cfg = engine_config_for(build_parser().parse_args(["m", "--kv-mem-gb", "4"]), block_bytes, 40960)
+    assert cfg.num_blocks == 2340 and cfg.max_model_len == 2340 * 16
+    small = engine_config_for(build_parser().parse_args(["m", "--kv-mem-gb", "1"]), block_bytes, 40960)
+    assert small.max_model_len == small.num_blocks * 16 < 40960
+    capped = engine_config_for(build_parser().parse_args(["m", "--kv-mem-gb", "64"]), block_bytes, 40960)
+    assert capped.max_model_len == 40960
+
+
+def test_bytes_per_block_of_a_model():
+    import torch
+
+    from atomserve_amd.cache import CachePools
+    from atomserve_amd.parts.base import PagedCacheRequest
+
+    requests = {i: PagedCacheRequest(8, 128) for i in range(28)}
+    assert CachePools.bytes_per_block(requests, 16, torch.bfloat16) == 28 * 2 * 8 * 128 * 2 * 16
+
+
+def test_prompt_ids_are_parsed():
+    assert parse_ids("1, 2,3  4") == [1, 2, 3, 4]
