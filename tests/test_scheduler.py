@@ -71,7 +71,8 @@ def run(prompts, params=GREEDY, **config):
     seqs = [Sequence(i, list(p), params) for i, p in enumerate(prompts)]
     for q in seqs:
         s.add(q)
-    return [q.output_ids for q in seqs], s, drive(s, runner)
+    preemptions = drive(s, runner)
+    return [q.output_ids for q in seqs], s, preemptions
 
 
 PROMPTS = [[1, 2, 3], [4, 5, 6, 7, 8, 9, 10], [11], [12, 13, 14, 15, 16], [17, 18]]
