@@ -64,15 +64,89 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const O* __restrict__ delt
   }
 }
 
+// The same with 16-byte accesses and the row kept in registers between the two passes:
+// every load of a row is in flight at once, which is what a decode step (few rows) needs.
+// Requires n % 4 == 0 and n <= 4 * blockDim.x * RN_CHUNKS.
+#define RN_CHUNKS 4
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ float4 load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+  static __device__ __forceinline__ void store(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <> struct Vec4<bf16> {
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ float4 load(const bf16* p) {
+    const bf16x4 r = *reinterpret_cast<const bf16x4*>(p);
+    return make_float4((float)r[0], (float)r[1], (float)r[2], (float)r[3]);
+  }
+  static __device__ __forceinline__ void store(bf16* p, float4 v) {
+    const bf16x4 r = {(bf16)v.x, (bf16)v.y, (bf16)v.z, (bf16)v.w};
+    *reinterpret_cast<bf16x4*>(p) = r;
+  }
+};
+
+template <typename O, typename W>
+__global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ x, const O* __restrict__ delta,
+                                                           const int* __restrict__ rows,
+                                                           const W* __restrict__ w, float eps,
+                                                           O* __restrict__ out, int n, int update_x) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = x + s * n;
+  const O* dr = delta ? delta + s * n : nullptr;
+  const int chunks = n >> 2;
+  float4 v[RN_CHUNKS];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < RN_CHUNKS; ++j) {
+    const int c = threadIdx.x + j * blockDim.x;
+    if (c < chunks) {
+      v[j] = Vec4<float>::load(xr + 4 * c);
+      if (dr) {
+        const float4 d = Vec4<O>::load(dr + 4 * c);
+        v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
+        if (update_x) Vec4<float>::store(xr + 4 * c, v[j]);
+      }
+      ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  O* o = out + (size_t)r * n;
+#pragma unroll
+  for (int j = 0; j < RN_CHUNKS; ++j) {
+    const int c = threadIdx.x + j * blockDim.x;
+    if (c < chunks) {
+      const float4 g = Vec4<W>::load(w + 4 * c);
+      Vec4<O>::store(o + 4 * c, make_float4(v[j].x * inv * g.x, v[j].y * inv * g.y, v[j].z * inv * g.z, v[j].w * inv * g.w));
+    }
+  }
+}
+
 extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const void* w, int w_dtype,
                           float eps, void* out, int out_dtype, int num_out_rows, int n, int update_x,
                           hipStream_t stream) {
   if (num_out_rows <= 0) return AS_OK;
   if (n <= 0) return AS_BAD_SHAPE;
-  const int threads = n >= 2048 ? 256 : (n >= 512 ? 128 : 64);
-#define LAUNCH(O, W)                                                                              \
-  rmsnorm_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)delta, rows, (const W*)w, \
-                                                             eps, (O*)out, n, update_x)
+  const bool vec = (n & 3) == 0 && n <= 4 * 1024 * RN_CHUNKS;
+  int threads = n >= 2048 ? 256 : (n >= 512 ? 128 : 64);
+  if (vec) {
+    // few rows: one chunk per thread, all loads in flight; many rows: fewer, fuller threads
+    const int chunks = n >> 2, per_thread = num_out_rows >= 512 ? RN_CHUNKS : 1;
+    threads = (chunks + per_thread - 1) / per_thread;
+    threads = ((threads + 63) / 64) * 64;
+    if (threads > 1024) threads = 1024;
+  }
+#define LAUNCH(O, W)                                                                               \
+  do {                                                                                             \
+    if (vec)                                                                                       \
+      rmsnorm_vec_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)delta, rows, (const W*)w, eps, \
+                                                                     (O*)out, n, update_x);        \
+    else                                                                                           \
+      rmsnorm_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)delta, rows, (const W*)w, eps,     \
+                                                                 (O*)out, n, update_x);            \
+  } while (0)
   if (out_dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
   else if (out_dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
   else if (out_dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);

@@ -90,17 +90,132 @@ __device__ __forceinline__ float exp1_noise(long long seed, int counter, int can
   return fmaxf(-logf(u), 1e-10f);
 }
 
+// The largest key among a thread's elements i = tid, tid + T, ...; four independent chains
+// keep several loads in flight.
+__device__ __forceinline__ unsigned long long thread_max_key(const float* __restrict__ x, int V) {
+  unsigned long long b0 = 0ull, b1 = 0ull, b2 = 0ull, b3 = 0ull;
+  const int T = blockDim.x;
+  int i = threadIdx.x;
+  for (; i + 3 * T < V; i += 4 * T) {
+    const float v0 = x[i], v1 = x[i + T], v2 = x[i + 2 * T], v3 = x[i + 3 * T];
+    const unsigned long long k0 = make_key(v0, i), k1 = make_key(v1, i + T), k2 = make_key(v2, i + 2 * T),
+                             k3 = make_key(v3, i + 3 * T);
+    b0 = k0 > b0 ? k0 : b0; b1 = k1 > b1 ? k1 : b1; b2 = k2 > b2 ? k2 : b2; b3 = k3 > b3 ? k3 : b3;
+  }
+  for (; i < V; i += T) { const unsigned long long k = make_key(x[i], i); b0 = k > b0 ? k : b0; }
+  b0 = b1 > b0 ? b1 : b0;
+  b2 = b3 > b2 ? b3 : b2;
+  return b2 > b0 ? b2 : b0;
+}
+
+// The k largest keys of a row in order, into sel[0..k-1]; returns how many were found (fewer
+// than k only if the row has fewer usable entries).  Block-wide; k <= SAMPLE_KMAX.
+//
+// 1. every thread finds the maximum of its own elements;
+// 2. t = the k-th largest of those 1024 maxima, by radix selection on the value bits: at
+//    least k elements are >= t, and usually few more;
+// 3. a second pass collects every element >= t into LDS;
+// 4. each candidate's rank is the number of candidates with a larger key.
+// If more candidates turn up than LDS holds (long runs of equal values), the slower
+// selection by repeated block-wide maximum takes over.
+#define SAMPLE_CAND 2048
+struct TopKShared {
+  unsigned long long red[17];
+  unsigned long long cand[SAMPLE_CAND];
+  unsigned int hist[256];
+  unsigned int count;
+  unsigned int prefix;
+  unsigned int remaining;
+};
+
+__device__ int block_topk(const float* __restrict__ x, int V, int k, unsigned long long* sel, TopKShared& sh) {
+  const int tid = threadIdx.x;
+  const unsigned long long mine = thread_max_key(x, V);
+  // radix selection of the k-th largest value (upper 32 bits of the key) among the thread maxima
+  const unsigned int myval = (unsigned int)(mine >> 32);
+  unsigned int prefix = 0, mask = 0;
+  int want = k;  // the want-th largest among the values matching the prefix
+  const int have = __syncthreads_count(mine != 0ull);
+  if (have < k) want = have;  // fewer than k usable maxima: take them all (t becomes the smallest)
+  if (want > 0) {
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      if (tid < 256) sh.hist[tid] = 0;
+      __syncthreads();
+      if (mine != 0ull && (myval & mask) == prefix) atomicAdd(&sh.hist[(myval >> shift) & 255], 1u);
+      __syncthreads();
+      if (tid == 0) {
+        int acc = 0, b = 255;
+        for (; b > 0; --b) {
+          if (acc + (int)sh.hist[b] >= want) break;
+          acc += sh.hist[b];
+        }
+        sh.prefix = prefix | ((unsigned int)b << shift);
+        sh.remaining = want - acc;
+      }
+      __syncthreads();
+      prefix = sh.prefix;
+      want = sh.remaining;
+      mask |= 255u << shift;
+    }
+  }
+  const unsigned int threshold = prefix;
+  if (tid == 0) sh.count = 0;
+  __syncthreads();
+  if (have > 0) {
+    const int T = blockDim.x;
+    for (int i0 = tid; i0 < V; i0 += 4 * T) {
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = (i0 + u * T < V) ? x[i0 + u * T] : __builtin_nanf("");
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const unsigned long long key = make_key(v[u], i0 + u * T);
+        if (key != 0ull && (unsigned int)(key >> 32) >= threshold) {
+          const unsigned int at = atomicAdd(&sh.count, 1u);
+          if (at < SAMPLE_CAND) sh.cand[at] = key;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const int count = sh.count;
+  if (count <= SAMPLE_CAND) {
+    for (int c = tid; c < count; c += blockDim.x) {
+      const unsigned long long key = sh.cand[c];
+      int rank = 0;
+      for (int j = 0; j < count; ++j) rank += sh.cand[j] > key;
+      if (rank < k) sel[rank] = key;
+    }
+    __syncthreads();
+    return count < k ? count : k;
+  }
+  // fallback: repeated block-wide maximum; after each pick only its owner looks for its next
+  unsigned long long cand = mine;
+  int found = 0;
+  for (int r = 0; r < k; ++r) {
+    const unsigned long long best = block_max_u64(cand, sh.red);
+    if (best == 0ull) break;
+    if (tid == 0) sel[r] = best;
+    found = r + 1;
+    if (key_index(best) % (int)blockDim.x == tid) {
+      unsigned long long next = 0ull;
+      for (int i = tid; i < V; i += blockDim.x) {
+        const unsigned long long key = make_key(x[i], i);
+        if (key < best && key > next) next = key;
+      }
+      cand = next;
+    }
+  }
+  __syncthreads();
+  return found;
+}
+
 // ---- greedy -----------------------------------------------------------------------
 __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __restrict__ logits,
                                                                 int* __restrict__ out, int V) {
   __shared__ unsigned long long red[17];
   const float* x = logits + (size_t)blockIdx.x * V;
-  unsigned long long best = 0ull;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const unsigned long long k = make_key(x[i], i);
-    best = k > best ? k : best;
-  }
-  best = block_max_u64(best, red);
+  const unsigned long long best = block_max_u64(thread_max_key(x, V), red);
   if (threadIdx.x == 0) out[blockIdx.x] = best ? key_index(best) : 0;
 }
 
@@ -131,7 +246,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const long long* __restrict__ seeds, const int* __restrict__ counters,
     int* __restrict__ out) {
-  __shared__ unsigned long long red[17];
+  __shared__ TopKShared topk_shared;
+  unsigned long long* red = topk_shared.red;
   __shared__ float fred[17];
   __shared__ unsigned long long sel[SAMPLE_KMAX];
   __shared__ float ework[SAMPLE_KMAX];
@@ -146,29 +262,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const bool all = (k <= 0 || k >= V);
 
   if (!all) {
-    // The k largest in order, by repeated block-wide maximum; after each pick only the
-    // thread that owned it looks for its next candidate.
     if (k > SAMPLE_KMAX) k = SAMPLE_KMAX;  // refused on the host; never index outside
-    unsigned long long cand = 0ull;
-    for (int i = tid; i < V; i += SAMPLE_THREADS) {
-      const unsigned long long key = make_key(x[i], i);
-      cand = key > cand ? key : cand;
-    }
-    int found = 0;
-    for (int r = 0; r < k; ++r) {
-      const unsigned long long best = block_max_u64(cand, red);
-      if (best == 0ull) break;  // fewer than k usable entries
-      if (tid == 0) sel[r] = best;
-      found = r + 1;
-      if (key_index(best) % SAMPLE_THREADS == tid) {
-        unsigned long long next = 0ull;
-        for (int i = tid; i < V; i += SAMPLE_THREADS) {
-          const unsigned long long key = make_key(x[i], i);
-          if (key < best && key > next) next = key;
-        }
-        cand = next;
-      }
-    }
+    const int found = block_topk(x, V, k, sel, topk_shared);
     __syncthreads();
     if (tid == 0) {
       int choice = 0;
@@ -245,28 +340,13 @@ extern "C" int as_sample(const float* logits, int B, int V, const float* tempera
 // Sorted top-k of each row (values and indices), k <= SAMPLE_KMAX; exposed for tests and tools.
 __global__ __launch_bounds__(SAMPLE_THREADS) void topk_kernel(const float* __restrict__ logits, int V, int k,
                                                               float* __restrict__ values, int* __restrict__ indices) {
-  __shared__ unsigned long long red[17];
-  const int row = blockIdx.x, tid = threadIdx.x;
-  const float* x = logits + (size_t)row * V;
-  unsigned long long cand = 0ull;
-  for (int i = tid; i < V; i += SAMPLE_THREADS) {
-    const unsigned long long key = make_key(x[i], i);
-    cand = key > cand ? key : cand;
-  }
-  for (int r = 0; r < k; ++r) {
-    const unsigned long long best = block_max_u64(cand, red);
-    if (tid == 0) {
-      values[(size_t)row * k + r] = best ? key_value(best) : -__builtin_inff();
-      indices[(size_t)row * k + r] = best ? key_index(best) : -1;
-    }
-    if (best != 0ull && key_index(best) % SAMPLE_THREADS == tid) {
-      unsigned long long next = 0ull;
-      for (int i = tid; i < V; i += SAMPLE_THREADS) {
-        const unsigned long long key = make_key(x[i], i);
-        if (key < best && key > next) next = key;
-      }
-      cand = next;
-    }
+  __shared__ TopKShared topk_shared;
+  __shared__ unsigned long long sel[SAMPLE_KMAX];
+  const int row = blockIdx.x;
+  const int found = block_topk(logits + (size_t)row * V, V, k, sel, topk_shared);
+  for (int r = threadIdx.x; r < k; r += blockDim.x) {
+    values[(size_t)row * k + r] = r < found ? key_value(sel[r]) : -__builtin_inff();
+    indices[(size_t)row * k + r] = r < found ? key_index(sel[r]) : -1;
   }
 }
 

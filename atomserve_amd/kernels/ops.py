@@ -173,6 +173,9 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
+SKINNY_MAX_ROWS = 16  # up to here the bf16 product streams the weights through our own kernel
+
+
 def gemm(a, w, out) -> None:
     """out[M, N] = a[M, K] @ w[N, K]^T.  fp32: own kernel (true fp32).  bf16: own kernel for few
     rows, the library's matrix product otherwise; `out` may be bf16 or (few rows) fp32."""
@@ -187,12 +190,14 @@ def gemm(a, w, out) -> None:
         _check(out, "out", F32)
         call("as_gemm_f32", _ptr(a), _ptr(w), _ptr(out), M, N, K, _stream())
         return
-    if out.dtype == BF16:
-        torch.mm(a, w.t(), out=out)
-    elif out.dtype == F32:
-        out.copy_(torch.mm(a, w.t()))
-    else:
+    if out.dtype not in (BF16, F32):
         raise KernelError(f"gemm: unsupported output dtype {out.dtype}")
+    if M <= SKINNY_MAX_ROWS and K % 8 == 0:
+        call("as_gemm_bf16_skinny", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, 0, _stream())
+    elif out.dtype == BF16:
+        torch.mm(a, w.t(), out=out)
+    else:
+        out.copy_(torch.mm(a, w.t()))
 
 
 SAMPLE_MAX_TOP_K = 1024

@@ -42,7 +42,7 @@ def test_embed_gather(ops, dtype):
     assert torch.equal(out, pk.embed_gather(table, ids))
 
 
-@pytest.mark.parametrize("n", [96, 1000, 4096, 5120])
+@pytest.mark.parametrize("n", [96, 97, 1000, 4096, 5120, 20000])
 @pytest.mark.parametrize("rows", [1, 7, 300])
 def test_rmsnorm_fp32(ops, n, rows):
     torch.manual_seed(1)
