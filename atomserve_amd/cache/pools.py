@@ -1,7 +1,8 @@
 """The tensors behind the cache manager's ids.
 
 A paged group has one pool [caches in group, 2 (k, v), num_pages, KV, block_size, D]
-in the compute dtype: the block_size keys of one head in one page are contiguous.  It
+in the compute dtype: the block_size keys of one head in one page are contiguous;
+the value half of a page is stored transposed, [D, block_size].  It
 starts zeroed, so that no slot ever holds a non-finite value
 (reference atomserve/kv_cache.py:112-118).  A state group has
 [caches in group, max_num_seqs, *shape].
@@ -27,11 +28,15 @@ class CachePools:
             self.state.append(torch.zeros(shape, dtype=g.request.dtype, device=device))
 
     def pages(self, cache_id: int):
-        """(group index, k_pages, v_pages) of one cache; views [num_pages, KV, block_size, D]."""
+        """(group index, k_pages, v_pages) of one cache: k_pages [num_pages, KV, block_size, D];
+        v_pages [num_pages, KV, D, block_size], each page of values transposed so that the keys
+        of one coordinate are contiguous (what the matrix-core kernels read directly)."""
         kind, gi, li = self.manager.group_of_cache[cache_id]
         if kind != "paged":
             raise KeyError(f"cache {cache_id} is not paged")
-        return gi, self.paged[gi][li, 0], self.paged[gi][li, 1]
+        k = self.paged[gi][li, 0]
+        nb, kv, bs, d = k.shape
+        return gi, k, self.paged[gi][li, 1].view(nb, kv, d, bs)
 
     def state_of(self, cache_id: int):
         """(group index, state tensor [max_num_seqs, *shape]) of one cache."""

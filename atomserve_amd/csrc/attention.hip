@@ -1,8 +1,8 @@
 // Attention over the paged cache.
 //
-// Cache pages of one layer: k_pages, v_pages [num_pages, KV, block_size, D]; a token
-// at position p of a request lives in page table[p / block_size] at offset
-// p % block_size.  A query at position p sees the keys at positions lo..p, with
+// Cache pages of one layer: k_pages [num_pages, KV, block_size, D] and v_pages
+// [num_pages, KV, D, block_size] (values transposed within a page); a token at position p
+// of a request lives in page table[p / block_size] at offset p % block_size.  A query at position p sees the keys at positions lo..p, with
 // lo = max(0, p - window + 1) if window > 0, else 0.  Query head h reads kv head
 // h / (H / KV).  Scores, softmax and the weighted sum are fp32.
 //
@@ -108,9 +108,11 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
     float kv[CH], vv[CH];
     if (valid && active) {
       const int page = table[key / bs];
-      const size_t base = (((size_t)page * KV + kvh) * bs + key % bs) * D + j * CH;
-      Chunk<T>::load(k_pages + base, kv);
-      Chunk<T>::load(v_pages + base, vv);
+      const size_t head = ((size_t)page * KV + kvh) * bs * D;
+      Chunk<T>::load(k_pages + head + (size_t)(key % bs) * D + j * CH, kv);
+      const T* vt = v_pages + head + (size_t)(j * CH) * bs + key % bs;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) vv[c] = to_f32(vt[(size_t)c * bs]);
     } else {
 #pragma unroll
       for (int c = 0; c < CH; ++c) { kv[c] = 0.f; vv[c] = 0.f; }
@@ -218,6 +220,222 @@ __global__ void attn_reduce_kernel(const int* __restrict__ items, const float* _
     }
     out[((size_t)t * H + h) * D + d] = from_f32<T>(num / den);
   }
+}
+
+// ---- bf16 decode through the matrix cores ---------------------------------------------
+//
+// One workgroup (4 waves) per (query token, kv head, partition).  All G <= 16 query heads
+// of the group ride in the 16 columns of one MFMA tile, so every key and value is read
+// once for the whole group.  Per step a wave takes 32 keys (two tiles of 16):
+//
+//   S^T[key][head] = K[key][:] . Q[head][:]     A = keys, straight from the page (16 bytes
+//                                               per lane), B = queries, kept in registers
+//   online softmax per head on the accumulator layout (lane = head column)
+//   O^T[d][head]  += V^T[d][key] P^T[key][head] A = the transposed value page, straight from
+//                                               memory, B = P, which the lane already holds
+//
+// The softmax weights are rounded to bf16 for the second product; maxima, sums and the
+// output accumulate in fp32.  Needs D % 32 == 0, D <= 256, block_size % 16 == 0.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int DC>  // D / 32
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ items, const int* __restrict__ positions, const int* __restrict__ tok_row,
+    const int* __restrict__ block_tables, int table_width, bf16* __restrict__ out, float* __restrict__ part_m,
+    float* __restrict__ part_l, float* __restrict__ part_acc, int H, int KV, int bs, float scale, int window,
+    int part_size, int P) {
+  constexpr int D = DC * 32, DT = DC * 2;  // DT: tiles of 16 output coordinates
+  extern __shared__ float smem[];          // [4][16] m, [4][16] l, [4][D][G] acc
+  const int G = H / KV;
+  const int item = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
+  const int t = items[item];
+  const int pos = positions[t];
+  const int ctx = pos + 1;
+  const int lo = window > 0 ? max(0, ctx - window) : 0;
+  const int k0 = max(lo, part * part_size), k1 = min(ctx, (part + 1) * part_size);
+  const int h0 = kvh * G;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;  // col: head within the group (and key row of A)
+
+  if (k0 >= k1) {
+    if (tid < G) {
+      const size_t o = ((size_t)item * H + h0 + tid) * P + part;
+      part_m[o] = NEG_INF;
+      part_l[o] = 0.f;
+    }
+    return;
+  }
+  const int* table = block_tables + (size_t)tok_row[t] * table_width;
+
+  bf16x8_t qop[DC];
+  {
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bf16* qrow = q + ((size_t)t * H + h0 + min(col, G - 1)) * D + grp * 8;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) qop[c] = col < G ? *reinterpret_cast<const bf16x8_t*>(qrow + c * 32) : zero;
+  }
+  f32x4_t o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = NEG_INF, l = 0.f;
+
+  const int first = (k0 / 32) * 32;
+  for (int kb = first + 32 * wave; kb < k1; kb += 128) {
+    // ---- scores of 32 keys
+    f32x4_t s[2];
+    size_t vbase[2];
+    bool live[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key0 = kb + 16 * tt;
+      live[tt] = key0 < k1;
+      s[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      vbase[tt] = 0;
+      if (live[tt]) {
+        const int page = table[key0 / bs], off0 = key0 % bs;
+        const size_t head = ((size_t)page * KV + kvh) * bs * D;
+        const bf16* krow = k_pages + head + (size_t)(off0 + col) * D + grp * 8;
+        bf16x8_t kop[DC];
+#pragma unroll
+        for (int c = 0; c < DC; ++c) kop[c] = *reinterpret_cast<const bf16x8_t*>(krow + c * 32);
+#pragma unroll
+        for (int c = 0; c < DC; ++c) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[c], qop[c], s[tt], 0, 0, 0);
+        vbase[tt] = head + off0 + 4 * grp;
+      }
+    }
+    // ---- online softmax for this lane's head column
+    float mx = NEG_INF;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kb + 16 * tt + 4 * grp + r;
+        const bool seen = live[tt] && key >= k0 && key < k1;
+        s[tt][r] = seen ? s[tt][r] * scale : NEG_INF;
+        mx = fmaxf(mx, s[tt][r]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float mn = fmaxf(m, mx);
+    float alpha = 1.f, rs = 0.f;
+    bf16x8_t pop;
+    if (mn == NEG_INF) {  // nothing seen yet (a window may hide whole steps)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pop[j] = (bf16)0.f;
+    } else {
+      alpha = (m == NEG_INF) ? 0.f : __expf(m - mn);
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float pv = __expf(s[tt][r] - mn);  // exp(-inf) = 0 for hidden keys
+          rs += pv;
+          pop[tt * 4 + r] = (bf16)pv;
+        }
+      m = mn;
+    }
+    rs += __shfl_xor(rs, 16, WAVE);
+    rs += __shfl_xor(rs, 32, WAVE);
+    l = l * alpha + rs;
+    // ---- weighted values
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x8_t vop;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        bf16x4_t v4 = {0, 0, 0, 0};
+        if (live[tt]) v4 = *reinterpret_cast<const bf16x4_t*>(v_pages + vbase[tt] + (size_t)(dt * 16 + col) * bs);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
+      }
+      o[dt] *= alpha;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop, o[dt], 0, 0, 0);
+    }
+  }
+
+  // ---- merge the four waves
+  float* sm = smem;
+  float* sl = smem + 64;
+  float* so = smem + 128;  // [4][D][G]
+  if (grp == 0 && col < G) { sm[wave * 16 + col] = m; sl[wave * 16 + col] = l; }
+  if (col < G) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) so[((size_t)wave * D + dt * 16 + 4 * grp + r) * G + col] = o[dt][r];
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int g = idx / D, d = idx % D;
+    float mxw = NEG_INF;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mxw = fmaxf(mxw, sm[w * 16 + g]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = sm[w * 16 + g];
+      const float e = (mw == NEG_INF) ? 0.f : __expf(mw - mxw);
+      num += so[((size_t)w * D + d) * G + g] * e;
+      den += sl[w * 16 + g] * e;
+    }
+    const int h = h0 + g;
+    if (P == 1) {
+      out[((size_t)t * H + h) * D + d] = (bf16)(num / den);
+    } else {
+      const size_t ob = ((size_t)item * H + h) * P + part;
+      part_acc[ob * D + d] = num;
+      if (d == 0) { part_m[ob] = mxw; part_l[ob] = den; }
+    }
+  }
+}
+
+static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_pages, const int* items,
+                              int num_items, const int* positions, const int* tok_row, const int* block_tables,
+                              int table_width, void* out, float* part_m, float* part_l, float* part_acc, int H,
+                              int KV, int D, int bs, float scale, int window, int part_size, int P,
+                              hipStream_t stream) {
+  const int G = H / KV;
+  if (D % 32 || D > 256 || G > 16 || bs % 16 || part_size % 32) return AS_BAD_SHAPE;
+  dim3 grid(num_items, KV, P);
+  const size_t shmem = sizeof(float) * (size_t)(128 + 4 * D * G);
+#define LAUNCH(DCV)                                                                                       \
+  attn_decode_mfma_kernel<DCV><<<grid, 256, shmem, stream>>>(                                             \
+      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, items, positions, tok_row, block_tables, \
+      table_width, (bf16*)out, part_m, part_l, part_acc, H, KV, bs, scale, window, part_size, P)
+  switch (D / 32) {
+    case 1: LAUNCH(1); break;
+    case 2: LAUNCH(2); break;
+    case 3: LAUNCH(3); break;
+    case 4: LAUNCH(4); break;
+    case 5: LAUNCH(5); break;
+    case 6: LAUNCH(6); break;
+    case 7: LAUNCH(7); break;
+    default: LAUNCH(8); break;
+  }
+#undef LAUNCH
+  if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
+  if (P > 1) {
+    attn_reduce_kernel<bf16><<<dim3(num_items, H), D >= 64 ? 64 : 32, 0, stream>>>(items, part_m, part_l, part_acc,
+                                                                                 (bf16*)out, H, D, P);
+  }
+  return launch_status();
+}
+
+// Same contract as as_attn_single_query, bf16 only, through the matrix cores.
+extern "C" int as_attn_decode_mfma(const void* q, const void* k_pages, const void* v_pages, const int* items,
+                                   int num_items, const int* positions, const int* tok_row,
+                                   const int* block_tables, int table_width, void* out, float* part_m,
+                                   float* part_l, float* part_acc, int H, int KV, int D, int bs, float scale,
+                                   int window, int part_size, int P, hipStream_t stream) {
+  if (num_items <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || H % KV || D <= 0 || bs <= 0 || part_size <= 0 || P <= 0 || table_width <= 0)
+    return AS_BAD_SHAPE;
+  if (P > 1 && (!part_m || !part_l || !part_acc)) return AS_BAD_SHAPE;
+  return launch_decode_mfma(q, k_pages, v_pages, items, num_items, positions, tok_row, block_tables, table_width,
+                            out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size, P, stream);
 }
 
 static int pow2ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }

@@ -199,8 +199,10 @@ extern "C" int as_rope_table(const int* positions, const double* inv_freq, float
 // One wave per (token, head slot) of qkv [T, H + 2 KV, D].  q and k heads: optional
 // RMSNorm over the head's D values with gains qw / kw, then rotation of the pairs
 // (i, i + R/2), i < R/2, by the token's angle; coordinates >= R pass unrotated.
-// q goes to q_out [T, H, D]; k and v go to the cache pages [num_pages, KV, bs, D] at
-// slot = page * bs + offset.  v is copied as it is.  store_kv = 0 computes q only.
+// q goes to q_out [T, H, D]; k goes to k_pages [num_pages, KV, bs, D] and v, copied as it
+// is, to v_pages [num_pages, KV, D, bs] (each page of values is stored transposed, so that
+// the keys of one coordinate are contiguous), at slot = page * bs + offset.
+// store_kv = 0 computes q only.
 // Plain reference: reference atomserve/kernels.py:74-145, atomserve/model.py:326-333.
 template <typename O, typename W>
 __global__ void qk_norm_rope_store_kernel(const O* __restrict__ qkv, const W* __restrict__ qw,
@@ -218,12 +220,13 @@ __global__ void qk_norm_rope_store_kernel(const O* __restrict__ qkv, const W* __
     const int slot = slots[t];
     if (slot < 0) return;  // this token's keys are not stored (whole wave returns)
     const int kvh = is_k ? hs - H : hs - H - KV;
-    O* pages = is_k ? k_pages : v_pages;
-    dst = pages + (((size_t)(slot / block_size) * KV + kvh) * block_size + slot % block_size) * D;
-  }
-  if (!is_q && !is_k) {
-    for (int i = lane; i < D; i += WAVE) dst[i] = src[i];
-    return;
+    const size_t head = (size_t)(slot / block_size) * KV + kvh;
+    if (!is_k) {  // values: transposed within the page
+      O* vt = v_pages + head * block_size * D + slot % block_size;
+      for (int i = lane; i < D; i += WAVE) vt[(size_t)i * block_size] = src[i];
+      return;
+    }
+    dst = k_pages + (head * block_size + slot % block_size) * D;
   }
   const W* w = is_q ? qw : kw;
   float inv = 1.0f;

@@ -84,7 +84,8 @@ def qk_norm_rope_store(qkv, q_weight, k_weight, cos_sin, slots, q_out, k_pages, 
                        num_kv_heads, eps, store_kv=True) -> None:  # fmt: skip
     """Per-head norm (if weights are given), rotation (if `cos_sin` is given) and the cache store.
 
-    qkv [T, H + 2 KV, D]; q_out [T, H, D]; pages [num_pages, KV, block_size, D]; slots [T] int32
+    qkv [T, H + 2 KV, D]; q_out [T, H, D]; k_pages [num_pages, KV, block_size, D], v_pages
+    [num_pages, KV, D, block_size] (values transposed within a page); slots [T] int32
     (page * block_size + offset, or -1 for a token whose keys are not stored)."""
     _check(qkv, "qkv", (F32, BF16), (None, num_heads + 2 * num_kv_heads, None))
     T, _, D = qkv.shape
@@ -108,8 +109,8 @@ def qk_norm_rope_store(qkv, q_weight, k_weight, cos_sin, slots, q_out, k_pages, 
     if store_kv:
         _check(slots, "slots", I32, (T,))
         _check(k_pages, "k_pages", qkv.dtype, (None, num_kv_heads, None, D))
-        _check(v_pages, "v_pages", qkv.dtype, tuple(k_pages.shape))
         block_size = k_pages.shape[2]
+        _check(v_pages, "v_pages", qkv.dtype, (k_pages.shape[0], num_kv_heads, D, block_size))
     call("as_qk_norm_rope_store", _ptr(qkv), _DT[qkv.dtype], _ptr(q_weight), _ptr(k_weight), _DT[w_dtype],
          _ptr(cos_sin), _ptr(slots) if store_kv else 0, _ptr(q_out), _ptr(k_pages) if store_kv else 0,
          _ptr(v_pages) if store_kv else 0, T, num_heads, num_kv_heads, D, R, float(eps), block_size,
@@ -130,8 +131,10 @@ SINGLE_QUERY_MAX_HEAD_DIM = 256
 
 
 def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tables, out, scale, window,
-                      max_context, part_size=None) -> None:  # fmt: skip
-    """Attention of single query tokens over the paged cache.
+                      max_context, part_size=None, force_generic=False) -> None:  # fmt: skip
+    """Attention of single query tokens over the paged cache.  bfloat16 with head widths in steps
+    of 32, groups of up to 16 heads and pages of a multiple of 16 tokens runs on the matrix cores;
+    everything else (and all of fp32) on the general kernel.
 
     q, out [T, H, D]; items [N] int32: the tokens (rows of q) to process; positions, tok_row [T]
     int32; block_tables [R, W] int32; max_context: host bound on positions[items] + 1."""
@@ -139,8 +142,8 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
     T, H, D = q.shape
     _check(out, "out", q.dtype, (T, H, D))
     _check(k_pages, "k_pages", q.dtype, (None, None, None, D))
-    _check(v_pages, "v_pages", q.dtype, tuple(k_pages.shape))
     _, KV, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", q.dtype, (k_pages.shape[0], KV, D, bs))
     _check(items, "items", I32, (None,))
     _check(positions, "positions", I32, (T,))
     _check(tok_row, "tok_row", I32, (T,))
@@ -155,19 +158,32 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
     span = min(max_context, window) if window > 0 else max_context
+    G = H // KV
+    mfma = q.dtype == BF16 and D % 32 == 0 and G <= 16 and bs % 16 == 0 and not force_generic
     if part_size is None:
-        # Enough partitions to occupy the GPU when few tokens are in the batch, few enough
-        # that the merge stays small; boundaries are multiples of part_size in absolute position.
-        groups = N * KV * max(1, (H // KV + 7) // 8)
-        part_size = 256
-        while part_size < span and groups * math.ceil(span / part_size) > 2048:
+        # Enough partitions to occupy the GPU when few tokens are in the batch, few enough that
+        # the merge stays small; boundaries are multiples of part_size in absolute position.
+        if mfma:
+            groups, part_size = N * KV, 128
+            limit = 1024
+        else:
+            groups, part_size = N * KV * max(1, (G + 7) // 8), 256
+            limit = 2048
+        while part_size < span and groups * math.ceil(span / part_size) > limit:
             part_size *= 2
+    if mfma and part_size % 32:
+        raise KernelError("attention: partitions of the matrix-core kernel are multiples of 32 keys")
     P = max(1, math.ceil(max_context / part_size))
     part_m = part_l = part_acc = None
     if P > 1:
         part_m = torch.empty((N, H, P), dtype=F32, device=q.device)
         part_l = torch.empty((N, H, P), dtype=F32, device=q.device)
         part_acc = torch.empty((N, H, P, D), dtype=F32, device=q.device)
+    if mfma:
+        call("as_attn_decode_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, _ptr(positions),
+             _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
+             _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+        return
     call("as_attn_single_query", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(items), N,
          _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m),
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip

@@ -48,20 +48,23 @@ def qk_norm_rope(qkv, q_weight, k_weight, cos_sin, num_heads, num_kv_heads, eps)
 
 
 def store_pages(k_pages, v_pages, k, v, slots):
-    """Write k, v [T, KV, D] into pages [P, KV, bs, D] at slot = page * bs + offset (slot < 0: skip)."""
+    """Write k, v [T, KV, D] at slot = page * bs + offset (slot < 0: skip) into k_pages
+    [P, KV, bs, D] and v_pages [P, KV, D, bs] (values transposed within a page)."""
     bs = k_pages.shape[2]
     for t, slot in enumerate(slots.tolist()):
         if slot < 0:
             continue
         k_pages[slot // bs, :, slot % bs, :] = k[t].to(k_pages.dtype)
-        v_pages[slot // bs, :, slot % bs, :] = v[t].to(v_pages.dtype)
+        v_pages[slot // bs, :, :, slot % bs] = v[t].to(v_pages.dtype)
 
 
-def gather_context(pages, table, length):
-    """Keys or values of positions 0..length-1 of one request: [length, KV, D]."""
-    bs = pages.shape[2]
+def gather_context(pages, table, length, transposed=False):
+    """Keys (or, transposed, values) of positions 0..length-1 of one request: [length, KV, D]."""
+    bs = pages.shape[3] if transposed else pages.shape[2]
     idx = torch.arange(length, device=pages.device)
     page = torch.as_tensor(table, device=pages.device).long()[idx // bs]
+    if transposed:
+        return pages[page, :, :, idx % bs]
     return pages[page, :, idx % bs, :]
 
 
@@ -76,7 +79,7 @@ def paged_attention(q, k_pages, v_pages, items, positions, tok_row, block_tables
         p = int(positions[t])
         table = block_tables[int(tok_row[t])]
         k = gather_context(k_pages, table, p + 1).double()
-        v = gather_context(v_pages, table, p + 1).double()
+        v = gather_context(v_pages, table, p + 1, transposed=True).double()
         lo = max(0, p - window + 1) if window > 0 else 0
         for h in range(H):
             s = (k[lo:, h // group, :] @ q[t, h].double()) * scale

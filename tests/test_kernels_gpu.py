@@ -112,11 +112,11 @@ def test_qk_norm_rope_store(ops, dtype, heads, D, bs):
     ops.rope_table(pos, inv, cs)
     pages = 64 // bs
     k_pages = torch.zeros(pages, KV, bs, D, dtype=dtype, device=DEV)
-    v_pages = torch.zeros_like(k_pages)
+    v_pages = torch.zeros(pages, KV, D, bs, dtype=dtype, device=DEV)
     q = torch.empty(5, H, D, dtype=dtype, device=DEV)
     ops.qk_norm_rope_store(qkv, qw, kw, cs, slots, q, k_pages, v_pages, H, KV, 1e-6)
     rq, rk, rv = pk.qk_norm_rope(qkv, qw, kw, cs, H, KV, 1e-6)
-    ref_k, ref_v = torch.zeros(pages, KV, bs, D, device=DEV), torch.zeros(pages, KV, bs, D, device=DEV)
+    ref_k, ref_v = torch.zeros(pages, KV, bs, D, device=DEV), torch.zeros(pages, KV, D, bs, device=DEV)
     pk.store_pages(ref_k, ref_v, rk, rv, slots)
     if dtype == F32:
         assert torch.allclose(q, rq, atol=1e-5) and torch.allclose(k_pages, ref_k, atol=1e-5)
@@ -136,7 +136,7 @@ def test_qk_norm_rope_store_variants(ops):
     inv = (1.0 / (1e4 ** (torch.arange(0, 16, 2, dtype=torch.float64) / 16))).to(DEV)
     cs = torch.empty(3, 8, 2, device=DEV)
     ops.rope_table(pos, inv, cs)
-    k_pages, v_pages = torch.zeros(2, KV, 8, D, device=DEV), torch.zeros(2, KV, 8, D, device=DEV)
+    k_pages, v_pages = torch.zeros(2, KV, 8, D, device=DEV), torch.zeros(2, KV, D, 8, device=DEV)
     q = torch.empty(3, H, D, device=DEV)
     ops.qk_norm_rope_store(qkv, None, None, cs, slots, q, k_pages, v_pages, H, KV, 0.0)
     rq, rk, rv = pk.qk_norm_rope(qkv, None, None, cs, H, KV, 0.0)
@@ -203,7 +203,7 @@ def paged_case(dtype, H, KV, D, bs, lens, seed=0, k_scale=4.0):
     g = torch.Generator().manual_seed(seed)
     pages = sum(-(-n // bs) for n in lens) + 8
     k_pages = (torch.randn(pages, KV, bs, D, generator=g) * k_scale).to(dtype).to(DEV)
-    v_pages = torch.randn(pages, KV, bs, D, generator=g).to(dtype).to(DEV)
+    v_pages = torch.randn(pages, KV, D, bs, generator=g).to(dtype).to(DEV)  # values transposed within a page
     perm = torch.randperm(pages, generator=g).tolist()
     tables, at = [], 0
     for n in lens:
@@ -232,13 +232,14 @@ def test_attention_single_query(ops, dtype, H, KV, D, bs):
     out = torch.zeros(len(lens), H, D, dtype=dtype, device=DEV)
     scale = D**-0.5
     ref = pk.paged_attention(q, k_pages, v_pages, items, positions, rows, tables, scale)
-    for part_size in (None, 256, 64):
+    for part_size, generic in ((None, False), (256, False), (64, False), (None, True), (64, True)):
         out.zero_()
-        ops.attn_single_query(q, k_pages, v_pages, items, positions, rows, tables, out, scale, 0, max(lens), part_size)
+        ops.attn_single_query(q, k_pages, v_pages, items, positions, rows, tables, out, scale, 0, max(lens), part_size,
+                              force_generic=generic)  # fmt: skip
         if dtype == F32:
             assert torch.allclose(out, ref, atol=1e-5), f"partitions of {part_size}: {(out - ref).abs().max()}"
         else:
-            assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), f"{(out.float() - ref).abs().max()}"
+            assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), f"{part_size, generic}: {(out.float() - ref).abs().max()}"
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -252,23 +253,26 @@ def test_attention_finds_one_far_key_among_many(ops, dtype):
         G = H // KV
         for kvh in range(KV):  # the first query head of each group gets its match
             k_pages[page, kvh, off] = (q[0, kvh * G].float() * 4.0).to(dtype)
-        out = torch.zeros(1, H, D, dtype=dtype, device=DEV)
-        ops.attn_single_query(q, k_pages, v_pages, i32([0]), positions, i32([0]), tables, out, 1.0, 0, n)
-        for kvh in range(KV):
-            want = v_pages[page, kvh, off].float()
-            assert torch.allclose(out[0, kvh * G].float(), want, atol=2e-2), (far, kvh)
+        for generic in (False, True):
+            out = torch.zeros(1, H, D, dtype=dtype, device=DEV)
+            ops.attn_single_query(q, k_pages, v_pages, i32([0]), positions, i32([0]), tables, out, 1.0, 0, n,
+                                  force_generic=generic)  # fmt: skip
+            for kvh in range(KV):
+                want = v_pages[page, kvh, :, off].float()
+                assert torch.allclose(out[0, kvh * G].float(), want, atol=2e-2), (far, kvh, generic)
 
 
 @pytest.mark.parametrize("window", [1, 5, 16, 17, 300])
-def test_attention_window_edge(ops, window):
-    H, KV, D, bs = 4, 2, 32, 8
+@pytest.mark.parametrize("dtype,bs", [(F32, 8), (BF16, 16)])
+def test_attention_window_edge(ops, window, dtype, bs):
+    H, KV, D = 4, 2, 32
     lens = [1, 9, 100, 513]
-    q, k_pages, v_pages, tables, positions = paged_case(F32, H, KV, D, bs, lens)
+    q, k_pages, v_pages, tables, positions = paged_case(dtype, H, KV, D, bs, lens)
     items = rows = i32(list(range(4)))
-    out = torch.zeros(4, H, D, device=DEV)
+    out = torch.zeros(4, H, D, dtype=dtype, device=DEV)
     ops.attn_single_query(q, k_pages, v_pages, items, positions, rows, tables, out, D**-0.5, window, max(lens), 64)
     ref = pk.paged_attention(q, k_pages, v_pages, items, positions, rows, tables, D**-0.5, window)
-    assert torch.allclose(out, ref, atol=1e-5)
+    assert torch.allclose(out.float(), ref, atol=1e-5 if dtype == F32 else 2e-2)
 
 
 def test_attention_serves_only_the_listed_tokens(ops):
@@ -296,7 +300,7 @@ def test_kernels_refuse_what_they_cannot_do(ops):
         ops.rmsnorm(x.cpu(), torch.ones(8), 1e-6, torch.empty(2, 8))
     q = torch.zeros(1, 2, 6, device=DEV)
     with pytest.raises(KernelError, match="head width"):
-        ops.attn_single_query(q, torch.zeros(1, 1, 4, 6, device=DEV), torch.zeros(1, 1, 4, 6, device=DEV), i32([0]),
+        ops.attn_single_query(q, torch.zeros(1, 1, 4, 6, device=DEV), torch.zeros(1, 1, 6, 4, device=DEV), i32([0]),
                               i32([0]), i32([0]), i32([[0]]), torch.zeros_like(q), 1.0, 0, 1)  # fmt: skip
 
 
