@@ -392,6 +392,183 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   }
 }
 
+// ---- bf16 prefill through the matrix cores ----------------------------------------------
+//
+// Work item: up to 64 consecutive query tokens of one request (`tiles` rows: first flat
+// token, count, block-table row, position of the first) for one kv head.  A wave owns 32
+// of those queries for one query head, as two MFMA column tiles of 16; the waves of a
+// workgroup take the heads of the group, so they walk the same keys at about the same time
+// and share them in the cache.  Keys and values come straight from the pages, as in the
+// decode kernel, already holding this step's own tokens; a query at position p sees keys
+// lo..p by absolute position, wherever the row starts.
+template <int DC>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ tiles, const int* __restrict__ block_tables, int table_width,
+    bf16* __restrict__ out, int H, int KV, int bs, float scale, int window) {
+  constexpr int D = DC * 32, DT = DC * 2;
+  const int G = H / KV;
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int unit = blockIdx.z * 4 + wave;  // (half of the tile, head of the group)
+  if (unit >= 2 * G) return;
+  const int half = unit / G, head = kvh * G + unit % G;
+  const int tok0 = tiles[4 * tile], count = tiles[4 * tile + 1], row = tiles[4 * tile + 2];
+  const int pos0 = tiles[4 * tile + 3];
+  const int q0 = half * 32;  // first query of this wave within the tile
+  if (q0 >= count) return;
+  const int nq = min(32, count - q0);
+  const int* table = block_tables + (size_t)row * table_width;
+
+  bf16x8_t qop[2][DC];
+  int qpos[2];
+  bool qok[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const int qi = qt * 16 + col;
+    qok[qt] = qi < nq;
+    const int qc = min(qi, nq - 1);  // columns past the end repeat the last query and are not stored
+    qpos[qt] = pos0 + q0 + qc;
+    const bf16* qrow = q + ((size_t)(tok0 + q0 + qc) * H + head) * D + grp * 8;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) qop[qt][c] = *reinterpret_cast<const bf16x8_t*>(qrow + c * 32);
+  }
+  f32x4_t o[2][DT];
+  float m[2], l[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    m[qt] = NEG_INF;
+    l[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int last = pos0 + q0 + nq - 1;                                    // the last key any query here sees
+  const int lo_all = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;   // the first key any query here sees
+  for (int kb = (lo_all / 32) * 32; kb <= last; kb += 32) {
+    bf16x8_t kop[2][DC];
+    size_t vbase[2];
+    bool live[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key0 = kb + 16 * tt;
+      live[tt] = key0 <= last;
+      vbase[tt] = 0;
+      if (live[tt]) {
+        const int page = table[key0 / bs], off0 = key0 % bs;
+        const size_t hbase = ((size_t)page * KV + kvh) * bs * D;
+        const bf16* krow = k_pages + hbase + (size_t)(off0 + col) * D + grp * 8;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) kop[tt][c] = *reinterpret_cast<const bf16x8_t*>(krow + c * 32);
+        vbase[tt] = hbase + off0 + 4 * grp;
+      } else {
+#pragma unroll
+        for (int c = 0; c < DC; ++c) kop[tt][c] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+    bf16x8_t pop[2];
+    float alpha[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      f32x4_t sc[2];
+      float mx = NEG_INF;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        sc[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < DC; ++c) sc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[tt][c], qop[qt][c], sc[tt], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = kb + 16 * tt + 4 * grp + r;
+          const bool seen = key <= qpos[qt] && (window <= 0 || key > qpos[qt] - window);
+          sc[tt][r] = seen ? sc[tt][r] * scale : NEG_INF;
+          mx = fmaxf(mx, sc[tt][r]);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float mn = fmaxf(m[qt], mx);
+      float rs = 0.f;
+      alpha[qt] = 1.f;
+      if (mn == NEG_INF) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pop[qt][j] = (bf16)0.f;
+      } else {
+        alpha[qt] = (m[qt] == NEG_INF) ? 0.f : __expf(m[qt] - mn);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float pv = __expf(sc[tt][r] - mn);
+            rs += pv;
+            pop[qt][tt * 4 + r] = (bf16)pv;
+          }
+        m[qt] = mn;
+      }
+      rs += __shfl_xor(rs, 16, WAVE);
+      rs += __shfl_xor(rs, 32, WAVE);
+      l[qt] = l[qt] * alpha[qt] + rs;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x8_t vop;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        bf16x4_t v4 = {0, 0, 0, 0};
+        if (live[tt]) v4 = *reinterpret_cast<const bf16x4_t*>(v_pages + vbase[tt] + (size_t)(dt * 16 + col) * bs);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
+      }
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        o[qt][dt] *= alpha[qt];
+        o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt], o[qt][dt], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    if (!qok[qt]) continue;
+    const float inv = 1.0f / l[qt];
+    bf16* orow = out + ((size_t)(tok0 + q0 + qt * 16 + col) * H + head) * D + 4 * grp;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const bf16x4_t r4 = {(bf16)(o[qt][dt][0] * inv), (bf16)(o[qt][dt][1] * inv), (bf16)(o[qt][dt][2] * inv),
+                           (bf16)(o[qt][dt][3] * inv)};
+      *reinterpret_cast<bf16x4_t*>(orow + dt * 16) = r4;
+    }
+  }
+}
+
+// tiles: [num_tiles, 4] int32 (first flat token, count <= 64, block-table row, first position).
+extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, const int* tiles,
+                                    int num_tiles, const int* block_tables, int table_width, void* out, int H,
+                                    int KV, int D, int bs, float scale, int window, hipStream_t stream) {
+  if (num_tiles <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || H % KV || bs <= 0 || table_width <= 0) return AS_BAD_SHAPE;
+  const int G = H / KV;
+  if (D % 32 || D <= 0 || D > 256 || bs % 16) return AS_BAD_SHAPE;
+  dim3 grid(num_tiles, KV, (2 * G + 3) / 4);
+#define LAUNCH(DCV)                                                                                    \
+  attn_prefill_mfma_kernel<DCV><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,       \
+                                                          (const bf16*)v_pages, tiles, block_tables,  \
+                                                          table_width, (bf16*)out, H, KV, bs, scale, window)
+  switch (D / 32) {
+    case 1: LAUNCH(1); break;
+    case 2: LAUNCH(2); break;
+    case 3: LAUNCH(3); break;
+    case 4: LAUNCH(4); break;
+    case 5: LAUNCH(5); break;
+    case 6: LAUNCH(6); break;
+    case 7: LAUNCH(7); break;
+    default: LAUNCH(8); break;
+  }
+#undef LAUNCH
+  return launch_status();
+}
+
 static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_pages, const int* items,
                               int num_items, const int* positions, const int* tok_row, const int* block_tables,
                               int table_width, void* out, float* part_m, float* part_l, float* part_acc, int H,

@@ -189,6 +189,35 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
+def attn_prefill_supported(dtype, head_dim: int, block_size: int) -> bool:
+    """Whether `attn_prefill` takes this case; if not, the rows go through `attn_single_query`."""
+    return dtype == BF16 and head_dim % 32 == 0 and head_dim <= 256 and block_size % 16 == 0
+
+
+def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context) -> None:
+    """Causal attention of prompt portions over the paged cache, bfloat16, on the matrix cores.
+
+    tiles [Nt, 4] int32: (first flat token, count <= 64, block-table row, position of the first
+    token) of up to 64 consecutive tokens of one request; the keys of these tokens are already in
+    the pages.  max_context: host bound on the last position + 1 of any tile."""
+    _check(q, "q", BF16, (None, None, None))
+    T, H, D = q.shape
+    _check(out, "out", BF16, (T, H, D))
+    _check(k_pages, "k_pages", BF16, (None, None, None, D))
+    _, KV, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", BF16, (k_pages.shape[0], KV, D, bs))
+    _check(tiles, "tiles", I32, (None, 4))
+    _check(block_tables, "block_tables", I32, (None, None))
+    if tiles.shape[0] == 0:
+        return
+    if H % KV or not attn_prefill_supported(q.dtype, D, bs):
+        raise KernelError(f"prefill attention: unsupported heads {H}/{KV}, head width {D} or page size {bs}")
+    if max_context > block_tables.shape[1] * bs:
+        raise KernelError("attention: block tables are shorter than the longest context")
+    call("as_attn_prefill_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(tiles), tiles.shape[0],
+         _ptr(block_tables), block_tables.shape[1], _ptr(out), H, KV, D, bs, float(scale), int(window), _stream())  # fmt: skip
+
+
 SKINNY_MAX_ROWS = 16  # up to here the bf16 product streams the weights through our own kernel
 
 

@@ -72,9 +72,9 @@ class Attention(Mixer):
 
     def attend(self, q, out, step, cache) -> None:
         s = self.spec
-        # fp32: every token is a single query.  bf16: short rows as single queries, long rows
-        # through the prefill kernel.
-        if self.env.dtype == torch.float32 or not hasattr(ops, "attn_prefill"):
+        # fp32, and shapes the prefill kernel does not take: every token is a single query.
+        # Otherwise short rows are single queries and long rows go through the prefill kernel.
+        if not ops.attn_prefill_supported(self.env.dtype, s.head_dim, cache.block_size):
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
                                   cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
             return
@@ -82,8 +82,8 @@ class Attention(Mixer):
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.short_tokens, step.positions, step.tok_row,
                                   cache.block_tables, out, s.scale, s.window, step.max_short_context)  # fmt: skip
         if step.num_long_tiles:
-            ops.attn_prefill(q, cache.k_pages, cache.v_pages, step.long_tiles, step.positions, step.tok_row,
-                             cache.block_tables, out, s.scale, s.window)  # fmt: skip
+            ops.attn_prefill(q, cache.k_pages, cache.v_pages, step.long_tiles, cache.block_tables, out, s.scale,
+                             s.window, step.max_context)  # fmt: skip
 
 
 register("mixer", "attention", Attention)

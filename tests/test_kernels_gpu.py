@@ -290,6 +290,45 @@ def test_attention_serves_only_the_listed_tokens(ops):
     assert bool((out[[0, 2, 3]] == 9.0).all())
 
 
+@pytest.mark.parametrize("H,KV,D,bs,window", [(32, 8, 128, 16, 0), (6, 2, 32, 16, 0), (8, 8, 64, 32, 0), (4, 1, 96, 16, 0),
+                                               (16, 2, 128, 16, 0), (4, 2, 64, 16, 40), (4, 2, 64, 16, 1)])  # fmt: skip
+def test_attention_prefill(ops, H, KV, D, bs, window):
+    """Prompt portions that start at position 0 and after a cached prefix, of lengths around
+    the tile sizes (16, 32, 64), each query seeing keys up to its own position."""
+    torch.manual_seed(12)
+    rows = [(0, 70), (37, 9), (100, 64), (5, 130), (300, 33), (0, 16), (511, 17)]  # (start, new tokens)
+    lens = [a + n for a, n in rows]
+    _, k_pages, v_pages, tables, _ = paged_case(BF16, H, KV, D, bs, lens, seed=3, k_scale=2.0 / math.sqrt(D / 16))
+    T = sum(n for _, n in rows)
+    q = torch.randn(T, H, D, device=DEV).to(BF16)
+    positions, tok_row, tiles, flat = [], [], [], 0
+    for r, (start, n) in enumerate(rows):
+        positions += list(range(start, start + n))
+        tok_row += [r] * n
+        for q0 in range(0, n, 64):
+            tiles.append([flat + q0, min(64, n - q0), r, start + q0])
+        flat += n
+    out = torch.zeros(T, H, D, dtype=BF16, device=DEV)
+    ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, window, max(lens))
+    ref = pk.paged_attention(q, k_pages, v_pages, i32(list(range(T))), i32(positions), i32(tok_row), tables, D**-0.5, window)
+    assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), (out.float() - ref).abs().max()
+
+
+def test_attention_prefill_sees_a_far_key_and_not_the_future(ops):
+    H, KV, D, bs, n = 4, 2, 64, 16, 700
+    for far in (0, 17, 255, 256, 640):
+        q_unused, k_pages, v_pages, tables, _ = paged_case(BF16, H, KV, D, bs, [n], seed=far, k_scale=0.05)
+        q = torch.randn(n, H, D, device=DEV).to(BF16)
+        page, off = int(tables[0, far // bs]), far % bs
+        k_pages[page, 0, off] = (q[650, 0].float() * 4.0).to(BF16)  # query 650 of head 0 matches key `far`
+        fut_page, fut_off = int(tables[0, 651 // bs]), 651 % bs
+        k_pages[fut_page, 0, fut_off] = (q[650, 0].float() * 8.0).to(BF16)  # a stronger match, one step in the future
+        tiles = [[q0, min(64, n - q0), 0, q0] for q0 in range(0, n, 64)]
+        out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
+        ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, 1.0, 0, n)
+        assert torch.allclose(out[650, 0].float(), v_pages[page, 0, :, off].float(), atol=2e-2), far
+
+
 def test_kernels_refuse_what_they_cannot_do(ops):
     from atomserve_amd.kernels.lib import KernelError
 
