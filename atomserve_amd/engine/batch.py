@@ -23,6 +23,7 @@ class Row:
     tables: the request's block table in each paged group; must cover every new position
     want:   indices into `tokens` whose next-token logits are asked for
     state_slot: the request's slot in the fixed-size state tables, or -1
+    store:  False for a filler row whose keys must not be written anywhere
     """
 
     tokens: list
@@ -30,6 +31,7 @@ class Row:
     tables: list
     want: list = field(default_factory=list)
     state_slot: int = -1
+    store: bool = True
 
 
 def slot_of(block_table: list, position: int, block_size: int) -> int:
@@ -72,7 +74,10 @@ class StepBatch:
     """
 
     def __init__(self, rows, block_size: int, num_paged_groups: int, vocab_size: int, device, pools=None,
-                 staging=None):  # fmt: skip
+                 staging=None, table_width: int = 0, max_context: int = 0, into=None):  # fmt: skip
+        """table_width, max_context: lower bounds that make the layout of a step independent of
+        its rows (a step whose kernels were captured in a graph is replayed with new contents).
+        into: an earlier batch of identical layout whose device buffer receives this one's arrays."""
         if not rows:
             raise ValueError("a step needs at least one row")
         bs = block_size
@@ -80,7 +85,7 @@ class StepBatch:
         slots = [[] for _ in range(num_paged_groups)]
         short, tiles = [], []
         row_first, row_len, row_start, row_slots = [], [], [], []
-        widths = [1] * num_paged_groups
+        widths = [max(1, table_width)] * num_paged_groups
         flat = 0
         self.max_context = self.max_short_context = 0
         for r, row in enumerate(rows):
@@ -100,7 +105,10 @@ class StepBatch:
                 first_page, last_page = row.start // bs, (end - 1) // bs
                 if any(table[b] == RELEASED for b in range(first_page, last_page + 1)):
                     raise ValueError("block table has given back a page that this row writes")
-                slots[g].extend(table[p // bs] * bs + p % bs for p in range(row.start, end))
+                if row.store:
+                    slots[g].extend(table[p // bs] * bs + p % bs for p in range(row.start, end))
+                else:
+                    slots[g].extend([-1] * n)
                 widths[g] = max(widths[g], (end + bs - 1) // bs)
             tok.extend(row.tokens)
             pos.extend(range(row.start, end))
@@ -119,6 +127,8 @@ class StepBatch:
             row_slots.append(row.state_slot)
             flat += n
 
+        self.max_context = max(self.max_context, max_context)
+        self.max_short_context = max(self.max_short_context, max_context if short else 0)
         T, R = flat, len(rows)
         tables = []
         for g in range(num_paged_groups):
@@ -138,15 +148,24 @@ class StepBatch:
             fields.append((f"tables{g}", tables[g].reshape(-1)))
         arrays = [np.asarray(list(v) if not isinstance(v, np.ndarray) else v, dtype=np.int32) for _, v in fields]
         total = sum(a.size for a in arrays)
+        sizes = [a.size for a in arrays]
+        if into is not None and into.layout != sizes:
+            raise ValueError("this step does not have the layout of the batch it should replace")
         if staging is not None:
             host = staging.take(total)
         else:
             host = torch.empty(total, dtype=torch.int32, pin_memory=torch.device(device).type == "cuda")
-        np.concatenate(arrays, out=host.numpy()[:total]) if total else None
-        dev = host[:total].to(device, non_blocking=True)
+        if total:
+            np.concatenate(arrays, out=host.numpy()[:total])
+        if into is not None:
+            dev = into.device_buffer
+            dev.copy_(host[:total], non_blocking=True)
+        else:
+            dev = host[:total].to(device, non_blocking=True)
         if staging is not None:
             staging.sent()
         self._host = host  # alive until the copy has run
+        self.device_buffer, self.layout = dev, sizes
         offset, parts = 0, {}
         for (name, _), a in zip(fields, arrays):
             parts[name] = dev[offset : offset + a.size]

@@ -29,10 +29,78 @@ def rows_for(seqs, num_new_tokens) -> list:
     return rows
 
 
+def _bucket(n: int, steps) -> int:
+    for s in steps:
+        if n <= s:
+            return s
+    return 0
+
+
+class DecodeGraphs:
+    """Decode steps (every row brings one token) replayed as HIP graphs.
+
+    A decode step is some hundred small launches; issuing them from the host costs more than
+    running them.  For each (rows rounded up, context rounded up) one pass is captured; later
+    steps copy their integers into the captured step's buffer and replay it.  Rows that pad a
+    step to its bucket store nothing and their logits are dropped.  Only kernels of this
+    package are captured (up to GRAPH_MAX_ROWS rows the matrix products are our own too)."""
+
+    ROW_BUCKETS = (1, 2, 4, 8, 16)
+    CONTEXT_STEP = 1024
+
+    def __init__(self, runner):
+        self.runner = runner
+        self.graphs = {}
+
+    def eligible(self, rows) -> bool:
+        r = self.runner
+        return (
+            r.device.type == "cuda"
+            and not r.manager.state_groups
+            and 0 < len(rows) <= self.ROW_BUCKETS[-1]
+            and all(len(row.tokens) == 1 for row in rows)
+        )
+
+    def run(self, rows):
+        r = self.runner
+        bs = r.manager.block_size
+        n = _bucket(len(rows), self.ROW_BUCKETS)
+        longest = max(row.start + 1 for row in rows)
+        context = -(-longest // self.CONTEXT_STEP) * self.CONTEXT_STEP
+        width = -(-context // bs)
+        filler = Row([0], 0, [[0] for _ in r.manager.paged_groups], [], -1, store=False)
+        padded = [Row(row.tokens, row.start, row.tables, [0], row.state_slot) for row in rows] + [
+            Row(filler.tokens, 0, filler.tables, [0], -1, store=False) for _ in range(n - len(rows))
+        ]
+        key = (n, context)
+        entry = self.graphs.get(key)
+        if entry is None:
+            batch = r.prepare(padded, table_width=width, max_context=context)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                r.model.forward(batch)  # loads every library and warms the allocator before capture
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = r.model.forward(batch)
+            entry = self.graphs[key] = (graph, batch, logits)
+        else:
+            r.prepare(padded, table_width=width, max_context=context, into=entry[1])
+        graph, batch, logits = entry
+        graph.replay()
+        wanted = [i for i, row in enumerate(rows) if row.want]
+        if wanted == list(range(len(rows))):
+            return logits[: len(rows)]
+        return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)] if wanted else logits[:0]
+
+
 class ModelRunner:
     """Owns the model, the cache pools and the sampler; executes one step for a list of rows."""
 
-    def __init__(self, model, manager: CacheManager, pools: CachePools = None):
+    def __init__(self, model, manager: CacheManager, pools: CachePools = None, use_graphs: bool = True):
         self.model = model
         self.manager = manager
         self.device = model.env.device
@@ -40,14 +108,19 @@ class ModelRunner:
         self.sampler = Sampler(self.device)
         self.staging = Staging(self.device)
         self.vocab_size = model.plan.vocab_size
+        self.decode_graphs = DecodeGraphs(self) if use_graphs else None
 
-    def prepare(self, rows) -> StepBatch:
+    def prepare(self, rows, **layout) -> StepBatch:
         return StepBatch(rows, self.manager.block_size, len(self.manager.paged_groups), self.vocab_size,
-                         self.device, pools=self.pools, staging=self.staging)  # fmt: skip
+                         self.device, pools=self.pools, staging=self.staging, **layout)  # fmt: skip
 
     @torch.inference_mode()
     def step(self, rows) -> torch.Tensor:
         """Logits [sum of len(row.want), vocab] fp32, in the order of the rows and of `want`."""
+        if self.decode_graphs is not None and self.decode_graphs.eligible(rows):
+            if any(w != 0 for row in rows for w in row.want):
+                raise ValueError("a row wants logits at a place outside its tokens")
+            return self.decode_graphs.run(rows)
         batch = self.prepare(rows)
         return self.model.forward(batch)
 
