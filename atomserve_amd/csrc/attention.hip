@@ -70,6 +70,8 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
       part_m[o] = NEG_INF;
       part_l[o] = 0.f;
     }
+    for (int idx = tid; idx < ng * D; idx += 256)
+      part_acc[(((size_t)item * H + h0 + idx / D) * P + part) * D + idx % D] = 0.f;
     return;
   }
 
@@ -198,27 +200,36 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
 }
 
 // Merge the partitions of each (item, head): out = sum_p acc_p e^(m_p - M) / sum_p l_p e^(m_p - M).
+// One workgroup per (item, head), one thread per output coordinate; every thread derives the
+// weights itself (P small values, all loads independent), so there is one round of loads for
+// the weights and one for the sums.  Empty partitions carry m = -inf, l = 0 and acc = 0.
+#define REDUCE_MAX_P 64
 template <typename T>
-__global__ void attn_reduce_kernel(const int* __restrict__ items, const float* __restrict__ part_m,
-                                   const float* __restrict__ part_l, const float* __restrict__ part_acc,
-                                   T* __restrict__ out, int H, int D, int P) {
+__global__ __launch_bounds__(256) void attn_reduce_kernel(const int* __restrict__ items,
+                                                          const float* __restrict__ part_m,
+                                                          const float* __restrict__ part_l,
+                                                          const float* __restrict__ part_acc, T* __restrict__ out,
+                                                          int H, int D, int P) {
   const int item = blockIdx.x, h = blockIdx.y;
-  const size_t o = ((size_t)item * H + h) * P;
+  const size_t base = ((size_t)item * H + h) * P;
   float mx = NEG_INF;
-  for (int p = 0; p < P; ++p) mx = fmaxf(mx, part_m[o + p]);
+  for (int p = 0; p < P; ++p) mx = fmaxf(mx, part_m[base + p]);
   float den = 0.f;
   for (int p = 0; p < P; ++p) {
-    const float mp = part_m[o + p];
-    den += (mp == NEG_INF) ? 0.f : part_l[o + p] * fexp<T>(mp - mx);
+    const float mp = part_m[base + p];
+    den += (mp == NEG_INF) ? 0.f : part_l[base + p] * fexp<T>(mp - mx);
   }
+  const float inv = 1.0f / den;
   const int t = items[item];
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float num = 0.f;
+#pragma unroll 4
     for (int p = 0; p < P; ++p) {
-      const float mp = part_m[o + p];
-      if (mp != NEG_INF) num += part_acc[(o + p) * D + d] * fexp<T>(mp - mx);
+      const float mp = part_m[base + p];
+      const float wgt = (mp == NEG_INF) ? 0.f : fexp<T>(mp - mx);
+      num += part_acc[(base + p) * D + d] * wgt;
     }
-    out[((size_t)t * H + h) * D + d] = from_f32<T>(num / den);
+    out[((size_t)t * H + h) * D + d] = from_f32<T>(num * inv);
   }
 }
 
@@ -240,6 +251,45 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+// The keys and values of one step (32 keys = two tiles of 16) of one kv head, as the MFMA
+// operands of this lane: keys as rows of A (16 bytes of each key's head), values as the
+// transposed page gives them (4 keys of one coordinate).  A tile that starts at or beyond
+// `end` is not read and counts as zeros.  Loading the next step before computing the current
+// one keeps memory busy while the matrix cores work.
+template <int DC>
+struct KVStep {
+  bf16x8_t k[2][DC];
+  bf16x4_t v[2][2 * DC];
+  bool live[2];
+};
+
+template <int DC>
+__device__ __forceinline__ void load_kv_step(KVStep<DC>& st, const bf16* __restrict__ k_pages,
+                                             const bf16* __restrict__ v_pages, const int* __restrict__ table,
+                                             int kb, int end, int KV, int kvh, int bs, int col, int grp) {
+  constexpr int D = DC * 32, DT = DC * 2;
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const int key0 = kb + 16 * tt;
+    st.live[tt] = key0 < end;
+    if (st.live[tt]) {
+      const int page = table[key0 / bs], off0 = key0 % bs;
+      const size_t head = ((size_t)page * KV + kvh) * bs * D;
+      const bf16* krow = k_pages + head + (size_t)(off0 + col) * D + grp * 8;
+#pragma unroll
+      for (int c = 0; c < DC; ++c) st.k[tt][c] = *reinterpret_cast<const bf16x8_t*>(krow + c * 32);
+      const bf16* vcol = v_pages + head + off0 + 4 * grp + (size_t)col * bs;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) st.v[tt][dt] = *reinterpret_cast<const bf16x4_t*>(vcol + (size_t)dt * 16 * bs);
+    } else {
+#pragma unroll
+      for (int c = 0; c < DC; ++c) st.k[tt][c] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) st.v[tt][dt] = bf16x4_t{0, 0, 0, 0};
+    }
+  }
+}
+
 template <int DC>  // D / 32
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
@@ -260,12 +310,14 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;  // col: head within the group (and key row of A)
 
-  if (k0 >= k1) {
+  if (k0 >= k1) {  // an empty partition (P > 1 only): mark it so for the reduce
     if (tid < G) {
       const size_t o = ((size_t)item * H + h0 + tid) * P + part;
       part_m[o] = NEG_INF;
       part_l[o] = 0.f;
     }
+    for (int idx = tid; idx < G * D; idx += 256)
+      part_acc[(((size_t)item * H + h0 + idx / D) * P + part) * D + idx % D] = 0.f;
     return;
   }
   const int* table = block_tables + (size_t)tok_row[t] * table_width;
@@ -283,28 +335,19 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   float m = NEG_INF, l = 0.f;
 
   const int first = (k0 / 32) * 32;
-  for (int kb = first + 32 * wave; kb < k1; kb += 128) {
+  KVStep<DC> cur, nxt;
+  int kb = first + 32 * wave;
+  if (kb < k1) load_kv_step<DC>(cur, k_pages, v_pages, table, kb, k1, KV, kvh, bs, col, grp);
+  for (; kb < k1; kb += 128) {
+    const bool more = kb + 128 < k1;
+    if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 128, k1, KV, kvh, bs, col, grp);
     // ---- scores of 32 keys
     f32x4_t s[2];
-    size_t vbase[2];
-    bool live[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      const int key0 = kb + 16 * tt;
-      live[tt] = key0 < k1;
       s[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      vbase[tt] = 0;
-      if (live[tt]) {
-        const int page = table[key0 / bs], off0 = key0 % bs;
-        const size_t head = ((size_t)page * KV + kvh) * bs * D;
-        const bf16* krow = k_pages + head + (size_t)(off0 + col) * D + grp * 8;
-        bf16x8_t kop[DC];
 #pragma unroll
-        for (int c = 0; c < DC; ++c) kop[c] = *reinterpret_cast<const bf16x8_t*>(krow + c * 32);
-#pragma unroll
-        for (int c = 0; c < DC; ++c) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[c], qop[c], s[tt], 0, 0, 0);
-        vbase[tt] = head + off0 + 4 * grp;
-      }
+      for (int c = 0; c < DC; ++c) s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[tt][c], qop[c], s[tt], 0, 0, 0);
     }
     // ---- online softmax for this lane's head column
     float mx = NEG_INF;
@@ -313,7 +356,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = kb + 16 * tt + 4 * grp + r;
-        const bool seen = live[tt] && key >= k0 && key < k1;
+        const bool seen = cur.live[tt] && key >= k0 && key < k1;
         s[tt][r] = seen ? s[tt][r] * scale : NEG_INF;
         mx = fmaxf(mx, s[tt][r]);
       }
@@ -345,15 +388,13 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) {
       bf16x8_t vop;
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        bf16x4_t v4 = {0, 0, 0, 0};
-        if (live[tt]) v4 = *reinterpret_cast<const bf16x4_t*>(v_pages + vbase[tt] + (size_t)(dt * 16 + col) * bs);
+      for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
-      }
+        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = cur.v[tt][dt][r];
       o[dt] *= alpha;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop, o[dt], 0, 0, 0);
     }
+    if (more) cur = nxt;
   }
 
   // ---- merge the four waves
@@ -446,27 +487,12 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 
   const int last = pos0 + q0 + nq - 1;                                    // the last key any query here sees
   const int lo_all = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;   // the first key any query here sees
-  for (int kb = (lo_all / 32) * 32; kb <= last; kb += 32) {
-    bf16x8_t kop[2][DC];
-    size_t vbase[2];
-    bool live[2];
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const int key0 = kb + 16 * tt;
-      live[tt] = key0 <= last;
-      vbase[tt] = 0;
-      if (live[tt]) {
-        const int page = table[key0 / bs], off0 = key0 % bs;
-        const size_t hbase = ((size_t)page * KV + kvh) * bs * D;
-        const bf16* krow = k_pages + hbase + (size_t)(off0 + col) * D + grp * 8;
-#pragma unroll
-        for (int c = 0; c < DC; ++c) kop[tt][c] = *reinterpret_cast<const bf16x8_t*>(krow + c * 32);
-        vbase[tt] = hbase + off0 + 4 * grp;
-      } else {
-#pragma unroll
-        for (int c = 0; c < DC; ++c) kop[tt][c] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      }
-    }
+  KVStep<DC> cur, nxt;
+  int kb = (lo_all / 32) * 32;
+  load_kv_step<DC>(cur, k_pages, v_pages, table, kb, last + 1, KV, kvh, bs, col, grp);
+  for (; kb <= last; kb += 32) {
+    const bool more = kb + 32 <= last;
+    if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 32, last + 1, KV, kvh, bs, col, grp);
     bf16x8_t pop[2];
     float alpha[2];
 #pragma unroll
@@ -477,7 +503,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
       for (int tt = 0; tt < 2; ++tt) {
         sc[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < DC; ++c) sc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[tt][c], qop[qt][c], sc[tt], 0, 0, 0);
+        for (int c = 0; c < DC; ++c) sc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[tt][c], qop[qt][c], sc[tt], 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = kb + 16 * tt + 4 * grp + r;
@@ -514,18 +540,16 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) {
       bf16x8_t vop;
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        bf16x4_t v4 = {0, 0, 0, 0};
-        if (live[tt]) v4 = *reinterpret_cast<const bf16x4_t*>(v_pages + vbase[tt] + (size_t)(dt * 16 + col) * bs);
+      for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
-      }
+        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = cur.v[tt][dt][r];
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) {
         o[qt][dt] *= alpha[qt];
         o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt], o[qt][dt], 0, 0, 0);
       }
     }
+    if (more) cur = nxt;
   }
 
 #pragma unroll
@@ -595,8 +619,8 @@ static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_
 #undef LAUNCH
   if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
   if (P > 1) {
-    attn_reduce_kernel<bf16><<<dim3(num_items, H), D >= 64 ? 64 : 32, 0, stream>>>(items, part_m, part_l, part_acc,
-                                                                                 (bf16*)out, H, D, P);
+    attn_reduce_kernel<bf16><<<dim3(num_items, H), D <= 64 ? 64 : (D <= 128 ? 128 : 256), 0, stream>>>(
+        items, part_m, part_l, part_acc, (bf16*)out, H, D, P);
   }
   return launch_status();
 }
@@ -644,8 +668,8 @@ static int launch_single_query(const void* q, const void* k_pages, const void* v
 #undef LAUNCH
   if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
   if (P > 1) {
-    attn_reduce_kernel<T><<<dim3(num_items, H), D >= 64 ? 64 : 32, 0, stream>>>(items, part_m, part_l, part_acc,
-                                                                              (T*)out, H, D, P);
+    attn_reduce_kernel<T><<<dim3(num_items, H), D <= 64 ? 64 : (D <= 128 ? 128 : 256), 0, stream>>>(
+        items, part_m, part_l, part_acc, (T*)out, H, D, P);
   }
   return launch_status();
 }

@@ -164,7 +164,7 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
         # Enough partitions to occupy the GPU when few tokens are in the batch, few enough that
         # the merge stays small; boundaries are multiples of part_size in absolute position.
         if mfma:
-            groups, part_size = N * KV, 128
+            groups, part_size = N * KV, 128  # 4 waves x 32 keys: one round of loads per workgroup
             limit = 1024
         else:
             groups, part_size = N * KV * max(1, (G + 7) // 8), 256
