@@ -1,0 +1,346 @@
+"""Parts alone and composed: each part of a layer against its plain reference, and models
+that are not Qwen3, registered from here without a change to the package: a mixer with a
+fixed-size state of its own in some layers, a layer that runs twice, and a run that reads
+the cache another run wrote."""
+
+import dataclasses
+import math
+
+import pytest
+import torch
+
+from tests import plain_kernels as pk
+from tests import plain_qwen3 as plain
+from tests.conftest import TINY_A, TINY_B, plain_random_weights
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ---- a toy mixer, defined here ----------------------------------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class DecaySpec:
+    kind: str
+    hidden_size: int
+    decay: float
+
+
+def make_decay_mixer():
+    from atomserve_amd.parts.base import Mixer, StateCacheRequest, WeightDecl
+
+    class DecayMixer(Mixer):
+        """y_t = gain * s_t with s_t = decay * s_{t-1} + h_t: a running sum kept per request in a
+        fixed-size state slot, so a prompt cut anywhere continues where it stopped."""
+
+        def weight_decls(self):
+            return {"gain": WeightDecl((self.spec.hidden_size,), role="vector")}
+
+        def cache_request(self):
+            return StateCacheRequest((self.spec.hidden_size,), torch.float32)
+
+        def forward(self, h, step, cache):
+            out = torch.empty_like(h)
+            flat = 0
+            for row in step.host_rows:
+                n = len(row.tokens)
+                s = cache.state[row.state_slot]
+                if row.start == 0:
+                    s.zero_()
+                for t in range(flat, flat + n):
+                    s.mul_(self.spec.decay).add_(h[t].float())
+                    out[t] = (s * self.gain.float()).to(h.dtype)
+                flat += n
+            return out
+
+    return DecayMixer
+
+
+def register_toy_architecture():
+    """Qwen3's layers with the mixer of every odd layer replaced by the decay mixer."""
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+    from atomserve_amd.parts.base import register
+
+    register("mixer", "toy_decay", make_decay_mixer(), replace=True)
+    qwen = architecture_for(TINY_A)
+
+    def build_plan(c):
+        plan = qwen.build_plan(c)
+        layers = tuple(
+            dataclasses.replace(layer, mixer=DecaySpec("toy_decay", c.hidden_size, 0.5 + 0.1 * i)) if i % 2 else layer
+            for i, layer in enumerate(plan.layers)
+        )
+        return dataclasses.replace(plan, layers=layers)
+
+    def checkpoint_map(c):
+        names = {k: v for k, v in qwen.checkpoint_map(c).items()
+                 if not any(k.startswith(f"layers.{i}.mixer.") for i in range(1, c.num_layers, 2))}  # fmt: skip
+        for i in range(1, c.num_layers, 2):
+            names[f"layers.{i}.mixer.gain"] = [f"model.layers.{i}.decay.gain"]
+        return names
+
+    def checkpoint_shapes(c):
+        shapes = {k: v for k, v in qwen.checkpoint_shapes(c).items()
+                  if not any(k.startswith(f"model.layers.{i}.self_attn.") for i in range(1, c.num_layers, 2))}  # fmt: skip
+        for i in range(1, c.num_layers, 2):
+            shapes[f"model.layers.{i}.decay.gain"] = ((c.hidden_size,), "vector")
+        return shapes
+
+    return register_architecture(
+        Architecture("ToyDecayForCausalLM", qwen.parse_config, build_plan, checkpoint_map, checkpoint_shapes), replace=True
+    )
+
+
+def plain_toy_logits(raw, w, ids):
+    """The toy model, whole sequence, no cache, from the plain functions."""
+    cfg = plain.normalise_config(raw)
+    wd = {k: v.double() for k, v in w.items()}
+    ids = torch.as_tensor(ids)
+    pos = torch.arange(len(ids))
+    x = plain.embed(wd["model.embed_tokens.weight"], ids)
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        h = plain.rms_norm(x, wd[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+        if i % 2:
+            s, ys = torch.zeros_like(h[0]), []
+            for t in range(len(ids)):
+                s = (0.5 + 0.1 * i) * s + h[t]
+                ys.append(s * wd[p + "decay.gain"])
+            x = x + torch.stack(ys)
+        else:
+            x = x + plain.attention_layer(h, wd, p, cfg, pos)
+        h = plain.rms_norm(x, wd[p + "post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+        x = x + plain.swiglu(h, wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"], wd[p + "mlp.down_proj.weight"])
+    x = plain.rms_norm(x, wd["model.norm.weight"], cfg["rms_norm_eps"])
+    head = "model.embed_tokens.weight" if cfg["tie_word_embeddings"] else "lm_head.weight"
+    return (x @ wd[head].T).float()
+
+
+def build_engine(arch, raw, weights, dtype, device=DEV, **engine):
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.models.decoder import DecoderModel
+    from atomserve_amd.weights.loader import DictSource, bind_checkpoint
+
+    config = arch.parse_config(raw)
+    model = DecoderModel(arch.build_plan(config), dtype, device)
+    bind_checkpoint(model, arch, config, DictSource(weights))
+    cfg = {"block_size": 16, "num_blocks": 32, "max_model_len": 256, "max_num_seqs": 4, "max_num_batched_tokens": 64, **engine}
+    return create_engine(model, EngineConfig(**cfg))
+
+
+def step_rows(engine, caches, entries):
+    """entries: (name, tokens, want) -> logits; requests keep their pages and slots in `caches`."""
+    from atomserve_amd.engine.batch import Row
+
+    m = engine.scheduler.manager
+    rows = []
+    for name, tokens, want in entries:
+        rc, done = caches.setdefault(name, [m.new_request(), 0])
+        assert m.reserve(rc, done, len(tokens))
+        rows.append(Row(tokens, done, rc.tables, want, rc.state_slot))
+        caches[name][1] += len(tokens)
+    return engine.runner.step(rows).float().cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_mixer_with_state_of_its_own(dtype, device=DEV):
+    arch = register_toy_architecture()
+    raw = {**TINY_B, "architectures": ["ToyDecayForCausalLM"], "num_hidden_layers": 4}
+    w = plain_random_weights(raw, seed=5, std=0.2, gain_std=0.2)
+    for i in (1, 3):
+        for k in [k for k in w if k.startswith(f"model.layers.{i}.self_attn.")]:
+            del w[k]
+        w[f"model.layers.{i}.decay.gain"] = (1 + 0.2 * torch.randn(raw["hidden_size"])).bfloat16().float()
+    engine = build_engine(arch, raw, w, dtype, device)
+    manager = engine.scheduler.manager
+    assert len(manager.state_groups) == 1 and len(manager.paged_groups) == 1 and not manager.prefix_reuse_possible
+    assert manager.paged_groups[0].cache_ids == [0, 2] and manager.state_groups[0].cache_ids == [1, 3]
+    a = torch.randint(0, 1000, (45,), generator=torch.Generator().manual_seed(1)).tolist()
+    b = torch.randint(0, 1000, (23,), generator=torch.Generator().manual_seed(2)).tolist()
+    ref_a, ref_b = plain_toy_logits(raw, w, a), plain_toy_logits(raw, w, b)
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    caches = {}
+    whole = step_rows(engine, caches, [("a", a, list(range(45)))])
+    assert (whole - ref_a).abs().max() <= tol * max(1.0, ref_a.abs().max())
+    # the same request cut anywhere, beside another one: the state carries over between steps
+    caches2 = {}
+    got_a, got_b = [], []
+    got = step_rows(engine, caches2, [("a2", a[:10], list(range(10))), ("b", b[:2], [0, 1])])
+    got_a.append(got[:10]); got_b.append(got[10:])  # noqa: E702
+    got = step_rows(engine, caches2, [("b", b[2:20], list(range(18))), ("a2", a[10:11], [0])])
+    got_b.append(got[:18]); got_a.append(got[18:])  # noqa: E702
+    got = step_rows(engine, caches2, [("a2", a[11:45], list(range(34))), ("b", b[20:], [0, 1, 2])])
+    got_a.append(got[:34]); got_b.append(got[34:])  # noqa: E702
+    assert (torch.cat(got_a) - ref_a).abs().max() <= tol * max(1.0, ref_a.abs().max())
+    assert (torch.cat(got_b) - ref_b).abs().max() <= tol * max(1.0, ref_b.abs().max())
+    for rc, _ in list(caches.values()) + list(caches2.values()):
+        manager.release(rc)
+    assert manager.num_free == manager.num_blocks and manager.num_free_slots == 4
+    # and through the scheduler: greedy generation equals the plain model's
+    from atomserve_amd.engine.sequence import SamplingParams
+
+    if dtype == torch.float32:
+        outs = engine.generate([a[:7], b[:12]], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
+        for prompt, out in zip((a[:7], b[:12]), outs):
+            seq = list(prompt)
+            for t in out:
+                assert t == int(plain_toy_logits(raw, w, seq)[-1].argmax())
+                seq.append(t)
+
+
+def plain_looped_logits(raw, w, ids):
+    """Run list [0, 1, 1 again reading the cache of its first run]: the second run of layer 1
+    takes its queries from the current hidden state and its keys and values from the first run."""
+    cfg = plain.normalise_config(raw)
+    wd = {k: v.double() for k, v in w.items()}
+    ids = torch.as_tensor(ids)
+    pos = torch.arange(len(ids))
+    T, H, KV, D = len(ids), cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps, theta = cfg["rms_norm_eps"], cfg["rope_theta"]
+    x = plain.embed(wd["model.embed_tokens.weight"], ids)
+    kept = None
+    for layer, reuse in ((0, False), (1, False), (1, True)):
+        p = f"model.layers.{layer}."
+        h = plain.rms_norm(x, wd[p + "input_layernorm.weight"], eps)
+        q = plain.rope(plain.rms_norm((h @ wd[p + "self_attn.q_proj.weight"].T).view(T, H, D), wd[p + "self_attn.q_norm.weight"], eps), pos, theta)
+        if reuse:
+            k, v = kept
+        else:
+            k = plain.rope(plain.rms_norm((h @ wd[p + "self_attn.k_proj.weight"].T).view(T, KV, D), wd[p + "self_attn.k_norm.weight"], eps), pos, theta)
+            v = (h @ wd[p + "self_attn.v_proj.weight"].T).view(T, KV, D)
+            kept = (k, v)
+        o = plain.causal_attention(q, k, v, pos)
+        x = x + o.reshape(T, H * D) @ wd[p + "self_attn.o_proj.weight"].T
+        h = plain.rms_norm(x, wd[p + "post_attention_layernorm.weight"], eps)
+        x = x + plain.swiglu(h, wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"], wd[p + "mlp.down_proj.weight"])
+    x = plain.rms_norm(x, wd["model.norm.weight"], eps)
+    return (x @ wd["model.embed_tokens.weight"].T).float()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_layer_runs_twice_and_reads_the_cache_of_its_first_run(dtype, device=DEV):
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+    from atomserve_amd.parts.plan import Run
+
+    qwen = architecture_for(TINY_A)
+
+    def build_plan(c):
+        return dataclasses.replace(qwen.build_plan(c), run=(Run(0), Run(1), Run(1, cache=1, writes=False)))
+
+    arch = register_architecture(
+        Architecture("LoopedForCausalLM", qwen.parse_config, build_plan, qwen.checkpoint_map, qwen.checkpoint_shapes), replace=True
+    )
+    raw = {**TINY_A, "architectures": ["LoopedForCausalLM"]}
+    w = plain_random_weights(raw, seed=6, std=0.2, gain_std=0.2)
+    engine = build_engine(arch, raw, w, dtype, device)
+    assert engine.scheduler.manager.paged_groups[0].cache_ids == [0, 1]  # three runs, two caches
+    ids = torch.randint(0, 256, (40,), generator=torch.Generator().manual_seed(3)).tolist()
+    ref = plain_looped_logits(raw, w, ids)
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    caches = {}
+    got = [step_rows(engine, caches, [("a", ids[:21], list(range(21)))])]
+    got += [step_rows(engine, caches, [("a", [ids[i]], [0])]) for i in range(21, 30)]
+    got.append(step_rows(engine, caches, [("a", ids[30:], list(range(10)))]))
+    assert (torch.cat(got) - ref).abs().max() <= tol * max(1.0, ref.abs().max())
+
+
+# ---- each part alone ------------------------------------------------------------------------
+
+
+def env(dtype):
+    from atomserve_amd.parts.base import BuildEnv
+
+    return BuildEnv(dtype=dtype, device=torch.device(DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from atomserve_amd.parts.base import build
+    from atomserve_amd.parts.plan import NormSpec
+
+    norm = build("norm", NormSpec("rmsnorm", 200, 1e-5), env(dtype))
+    assert {k: v.shape for k, v in norm.weight_decls().items()} == {"weight": (200,)}
+    w = (torch.randn(200, device=DEV) * 0.2 + 1).to(dtype)
+    norm.bind({"weight": w})
+    x = torch.randn(9, 200, device=DEV)
+    delta = torch.randn(9, 200, device=DEV).to(dtype)
+    ref, new_x = pk.rmsnorm(x, w, 1e-5, delta)
+    x_work = x.clone()
+    out = norm.forward(x_work, delta)
+    assert out.dtype == dtype and torch.allclose(x_work, new_x, atol=1e-6)
+    assert torch.allclose(out.float(), ref, atol=1e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from atomserve_amd.parts.base import build
+    from atomserve_amd.parts.plan import GatedMLPSpec
+
+    ffn = build("feed_forward", GatedMLPSpec("gated_mlp", 96, 160, "silu"), env(dtype))
+    assert {k: v.shape for k, v in ffn.weight_decls().items()} == {"gate_up.weight": (320, 96), "down.weight": (96, 160)}
+    gate_up = (torch.randn(320, 96, device=DEV) * 0.1).to(dtype)
+    down = (torch.randn(96, 160, device=DEV) * 0.1).to(dtype)
+    ffn.bind({"gate_up.weight": gate_up, "down.weight": down})
+    h = torch.randn(21, 96, device=DEV).to(dtype)
+    out = ffn.forward(h, None)
+    ref = plain.swiglu(h.double(), gate_up[:160].double(), gate_up[160:].double(), down.double()).float()
+    assert (out.float() - ref).abs().max() <= (1e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(ref.abs().max()))
+    with pytest.raises(ValueError, match="activation"):
+        build("feed_forward", GatedMLPSpec("gated_mlp", 96, 160, "gelu"), env(dtype))
+
+
+def test_position_part_and_unknown_kinds():
+    from atomserve_amd.parts.base import build
+    from atomserve_amd.parts.plan import NormSpec, RotarySpec
+
+    class Step:
+        num_tokens, shared = 4, {}
+        positions = torch.tensor([0, 1, 77, 30000], dtype=torch.int32, device=DEV)
+
+    rope = build("position", RotarySpec("rope_half", 32, 1e6), env(torch.float32))
+    table = rope.prepare(Step)
+    ang = plain.rope_angles(Step.positions.cpu(), 32, 1e6)
+    assert torch.allclose(table[..., 0].cpu().double(), ang.cos(), atol=2e-7) and torch.allclose(table[..., 1].cpu().double(), ang.sin(), atol=2e-7)
+    assert rope.prepare(Step) is table  # computed once per step, shared by the layers
+    with pytest.raises(ValueError, match="no norm part of kind"):
+        build("norm", NormSpec("layernorm", 8, 1e-5), env(torch.float32))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_part_alone(dtype):
+    """One attention mixer, built from its spec alone, against the plain attention layer: a
+    whole prompt, then the same prompt continued token by token from the cache."""
+    from atomserve_amd.cache import CacheManager, CachePools
+    from atomserve_amd.engine.batch import Row, StepBatch
+    from atomserve_amd.parts.base import build
+    from atomserve_amd.parts.plan import AttentionSpec, NormSpec, RotarySpec
+
+    h, H, KV, D = 80, 5, 1, 32
+    spec = AttentionSpec("attention", h, H, KV, D, 1 / math.sqrt(D), NormSpec("rmsnorm", D, 1e-5), RotarySpec("rope_half", D, 5e4))
+    mixer = build("mixer", spec, env(dtype))
+    torch.manual_seed(7)
+    w = {"qkv.weight": torch.randn((H + 2 * KV) * D, h) * 0.2, "o.weight": torch.randn(h, H * D) * 0.2,
+         "q_norm.weight": 1 + 0.2 * torch.randn(D), "k_norm.weight": 1 + 0.2 * torch.randn(D)}  # fmt: skip
+    w = {k: v.bfloat16().float() for k, v in w.items()}
+    mixer.bind({k: v.to(DEV).to(dtype) for k, v in w.items()})
+    manager = CacheManager({0: mixer.cache_request()}, 16, 8, 2)
+    pools = CachePools(manager, dtype, DEV)
+    x = torch.randn(30, h).bfloat16().float()
+    named = {"model.layers.0.self_attn.q_proj.weight": w["qkv.weight"][: H * D],
+             "model.layers.0.self_attn.k_proj.weight": w["qkv.weight"][H * D : (H + KV) * D],
+             "model.layers.0.self_attn.v_proj.weight": w["qkv.weight"][(H + KV) * D :],
+             "model.layers.0.self_attn.q_norm.weight": w["q_norm.weight"], "model.layers.0.self_attn.k_norm.weight": w["k_norm.weight"],
+             "model.layers.0.self_attn.o_proj.weight": w["o.weight"]}  # fmt: skip
+    cfg = {"num_attention_heads": H, "num_key_value_heads": KV, "head_dim": D, "rms_norm_eps": 1e-5, "rope_theta": 5e4}
+    ref = plain.attention_layer(x.double(), {k: v.double() for k, v in named.items()}, "model.layers.0.", cfg, torch.arange(30)).float()
+    rc = manager.new_request()
+    outs, at = [], 0
+    for n in (20, 1, 1, 8):
+        manager.reserve(rc, at, n)
+        batch = StepBatch([Row([0] * n, at, rc.tables, [])], 16, 1, 10, DEV, pools=pools)
+        outs.append(mixer.forward(x[at : at + n].to(DEV).to(dtype), batch, batch.cache_view(0, True)).float().cpu())
+        at += n
+    tol = (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(ref.abs().max()))
+    assert (torch.cat(outs) - ref).abs().max() <= tol
