@@ -7,6 +7,8 @@ the wanted places.  It never changes a sequence: advancing and appending is the
 scheduler's work, so the same plan can be inspected or retried.
 """
 
+import gc
+
 import torch
 
 from atomserve_amd.cache.manager import CacheManager
@@ -84,8 +86,18 @@ class DecodeGraphs:
             torch.cuda.synchronize()
             batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                logits = r.model.forward(batch)
+            # No garbage collection while the stream is capturing: a collected object of an
+            # earlier engine (a graph, a tensor) would be destroyed in the middle of the capture,
+            # which the runtime answers by aborting the process.
+            gc.collect()
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    logits = r.model.forward(batch)
+            finally:
+                if collecting:
+                    gc.enable()
             entry = self.graphs[key] = (graph, batch, logits)
         else:
             r.prepare(padded, table_width=width, max_context=context, into=entry[1])
