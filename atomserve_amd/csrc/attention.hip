@@ -437,30 +437,56 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 //
 // Work item: up to 64 consecutive query tokens of one request (`tiles` rows: first flat
 // token, count, block-table row, position of the first) for one kv head.  A wave owns 32
-// of those queries for one query head, as two MFMA column tiles of 16; the waves of a
-// workgroup take the heads of the group, so they walk the same keys at about the same time
-// and share them in the cache.  Keys and values come straight from the pages, as in the
-// decode kernel, already holding this step's own tokens; a query at position p sees keys
-// lo..p by absolute position, wherever the row starts.
+// of those queries for one query head, as two MFMA column tiles of 16; the four waves of a
+// workgroup take heads of the same group (or the other half of the queries), so they all
+// need the same keys and values.  Those are brought into LDS once per workgroup, 32 keys
+// per step: a 16-key piece of a page is contiguous in memory both for keys and, thanks to
+// the transposed value pages, for values, so every thread copies 16 bytes.  The next step
+// is on its way from memory while the current one is computed (double-buffered LDS).
+// A query at position p sees keys lo..p by absolute position, wherever the row starts.
+#define PF_PAD 8  // bf16 elements of padding per key row in LDS: spreads the rows over the banks
+
 template <int DC>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ tiles, const int* __restrict__ block_tables, int table_width,
     bf16* __restrict__ out, int H, int KV, int bs, float scale, int window) {
   constexpr int D = DC * 32, DT = DC * 2;
+  constexpr int KROW = D + PF_PAD;               // elements per key row in LDS
+  constexpr int KTILE = 16 * KROW, VTILE = D * 16;  // elements per 16-key tile
+  constexpr int CHUNKS = 2 * D;                  // 16-byte chunks per tile (keys or values)
+  constexpr int PER = (CHUNKS + 255) / 256;      // chunks per thread per tile
+  __shared__ __attribute__((aligned(16))) bf16 lds_k[2][2][KTILE];
+  __shared__ __attribute__((aligned(16))) bf16 lds_v[2][2][VTILE];
+
   const int G = H / KV;
   const int tile = blockIdx.x, kvh = blockIdx.y;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int unit = blockIdx.z * 4 + wave;  // (half of the tile, head of the group)
-  if (unit >= 2 * G) return;
-  const int half = unit / G, head = kvh * G + unit % G;
   const int tok0 = tiles[4 * tile], count = tiles[4 * tile + 1], row = tiles[4 * tile + 2];
   const int pos0 = tiles[4 * tile + 3];
-  const int q0 = half * 32;  // first query of this wave within the tile
-  if (q0 >= count) return;
-  const int nq = min(32, count - q0);
   const int* table = block_tables + (size_t)row * table_width;
+
+  // the keys this workgroup walks: from the first key any of its waves sees to the last
+  int wg_lo = 0x7fffffff, wg_last = -1;
+  for (int u = blockIdx.z * 4; u < blockIdx.z * 4 + 4 && u < 2 * G; ++u) {
+    const int uq0 = (u / G) * 32;
+    if (uq0 >= count) continue;
+    wg_last = max(wg_last, pos0 + min(count, uq0 + 32) - 1);
+    wg_lo = min(wg_lo, window > 0 ? max(0, pos0 + uq0 - window + 1) : 0);
+  }
+  if (wg_last < 0) return;  // uniform over the workgroup
+
+  // this wave's queries
+  const int unit = blockIdx.z * 4 + wave;
+  const int half = unit / G, head = kvh * G + unit % G;
+  const int q0 = half * 32;
+  const bool working = unit < 2 * G && q0 < count;
+  const int nq = working ? min(32, count - q0) : 1;
+  const int my_last = working ? pos0 + q0 + nq - 1 : -1;
+  const int my_first_q = pos0 + q0;                  // position of this wave's first query
+  const float scale2 = scale * 1.4426950408889634f;  // scores are kept in base 2
+  const int my_lo = working ? (window > 0 ? max(0, pos0 + q0 - window + 1) : 0) : 0x7fffffff;
 
   bf16x8_t qop[2][DC];
   int qpos[2];
@@ -468,12 +494,17 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
     const int qi = qt * 16 + col;
-    qok[qt] = qi < nq;
+    qok[qt] = working && qi < nq;
     const int qc = min(qi, nq - 1);  // columns past the end repeat the last query and are not stored
     qpos[qt] = pos0 + q0 + qc;
-    const bf16* qrow = q + ((size_t)(tok0 + q0 + qc) * H + head) * D + grp * 8;
+    if (working) {
+      const bf16* qrow = q + ((size_t)(tok0 + q0 + qc) * H + head) * D + grp * 8;
 #pragma unroll
-    for (int c = 0; c < DC; ++c) qop[qt][c] = *reinterpret_cast<const bf16x8_t*>(qrow + c * 32);
+      for (int c = 0; c < DC; ++c) qop[qt][c] = *reinterpret_cast<const bf16x8_t*>(qrow + c * 32);
+    } else {
+#pragma unroll
+      for (int c = 0; c < DC; ++c) qop[qt][c] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    }
   }
   f32x4_t o[2][DT];
   float m[2], l[2];
@@ -485,71 +516,139 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  const int last = pos0 + q0 + nq - 1;                                    // the last key any query here sees
-  const int lo_all = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;   // the first key any query here sees
-  KVStep<DC> cur, nxt;
-  int kb = (lo_all / 32) * 32;
-  load_kv_step<DC>(cur, k_pages, v_pages, table, kb, last + 1, KV, kvh, bs, col, grp);
-  for (; kb <= last; kb += 32) {
-    const bool more = kb + 32 <= last;
-    if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 32, last + 1, KV, kvh, bs, col, grp);
-    bf16x8_t pop[2];
-    float alpha[2];
+  // ---- staging: registers <- memory, LDS <- registers
+  bf16x8_t rk[2][PER], rv[2][PER];
+  auto fetch = [&](int kb) {
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      f32x4_t sc[2];
-      float mx = NEG_INF;
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key0 = kb + 16 * tt;
+      const bool live = key0 <= wg_last;
+      size_t base = 0;
+      int off0 = 0;
+      if (live) {
+        const int page = table[key0 / bs];
+        off0 = key0 % bs;
+        base = ((size_t)page * KV + kvh) * bs * D;
+      }
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        sc[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < DC; ++c) sc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[tt][c], qop[qt][c], sc[tt], 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int key = kb + 16 * tt + 4 * grp + r;
-          const bool seen = key <= qpos[qt] && (window <= 0 || key > qpos[qt] - window);
-          sc[tt][r] = seen ? sc[tt][r] * scale : NEG_INF;
-          mx = fmaxf(mx, sc[tt][r]);
+      for (int i = 0; i < PER; ++i) {
+        const int c = tid + i * 256;
+        rk[tt][i] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        rv[tt][i] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (live && c < CHUNKS) {
+          // keys: chunk c = 8 coordinates (c % (D/8)) of key row c / (D/8)
+          rk[tt][i] = *reinterpret_cast<const bf16x8_t*>(k_pages + base + (size_t)(off0 + c / (D / 8)) * D + (c % (D / 8)) * 8);
+          // values: chunk c = 8 keys (c % 2) of coordinate row c / 2
+          rv[tt][i] = *reinterpret_cast<const bf16x8_t*>(v_pages + base + (size_t)(c / 2) * bs + off0 + (c % 2) * 8);
         }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-      const float mn = fmaxf(m[qt], mx);
-      float rs = 0.f;
-      alpha[qt] = 1.f;
-      if (mn == NEG_INF) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pop[qt][j] = (bf16)0.f;
-      } else {
-        alpha[qt] = (m[qt] == NEG_INF) ? 0.f : __expf(m[qt] - mn);
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float pv = __expf(sc[tt][r] - mn);
-            rs += pv;
-            pop[qt][tt * 4 + r] = (bf16)pv;
-          }
-        m[qt] = mn;
-      }
-      rs += __shfl_xor(rs, 16, WAVE);
-      rs += __shfl_xor(rs, 32, WAVE);
-      l[qt] = l[qt] * alpha[qt] + rs;
     }
+  };
+  auto stash = [&](int buf) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      bf16x8_t vop;
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int c = tid + i * 256;
+        if (c < CHUNKS) {
+          *reinterpret_cast<bf16x8_t*>(&lds_k[buf][tt][(c / (D / 8)) * KROW + (c % (D / 8)) * 8]) = rk[tt][i];
+          *reinterpret_cast<bf16x8_t*>(&lds_v[buf][tt][(c / 2) * 16 + (c % 2) * 8]) = rv[tt][i];
+        }
+      }
+  };
+
+  int kb = (wg_lo / 32) * 32;
+  fetch(kb);
+  stash(0);
+  __syncthreads();
+  for (int buf = 0; kb <= wg_last; kb += 32, buf ^= 1) {
+    const bool more = kb + 32 <= wg_last;
+    if (more) fetch(kb + 32);
+    if (working && kb <= my_last && kb + 31 >= my_lo) {
+      // raw scores of 32 keys x 32 queries; a key operand is read from LDS once for both query tiles
+      f32x4_t sc[2][2];
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) sc[qt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = cur.v[tt][dt][r];
+        for (int c = 0; c < DC; ++c) {
+          const bf16x8_t kop = *reinterpret_cast<const bf16x8_t*>(&lds_k[buf][tt][col * KROW + c * 32 + grp * 8]);
+#pragma unroll
+          for (int qt = 0; qt < 2; ++qt)
+            sc[qt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[qt][c], sc[qt][tt], 0, 0, 0);
+        }
+      // Only steps that touch the causal diagonal, the window's edge or the end of the context
+      // need a mask; the others see all 32 keys (uniform over the wave).
+      const bool masked = kb + 31 > my_first_q || (window > 0 && kb < my_last - window + 1);
+      bf16x8_t pop[2];
+      float alpha[2];
+      bool rescale = false;
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) {
-        o[qt][dt] *= alpha[qt];
-        o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt], o[qt][dt], 0, 0, 0);
+        if (masked) {
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int key = kb + 16 * tt + 4 * grp + r;
+              const bool seen = key <= qpos[qt] && (window <= 0 || key > qpos[qt] - window);
+              sc[qt][tt][r] = seen ? sc[qt][tt][r] : NEG_INF;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3])),
+                         fmaxf(fmaxf(sc[qt][1][0], sc[qt][1][1]), fmaxf(sc[qt][1][2], sc[qt][1][3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        // base-2 softmax: scale and log2(e) are folded into one factor (positive, so maxima agree)
+        const float mn = fmaxf(m[qt], mx * scale2);
+        float rs = 0.f;
+        alpha[qt] = 1.f;
+        if (mn == NEG_INF) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pop[qt][j] = (bf16)0.f;
+        } else {
+          alpha[qt] = __builtin_amdgcn_exp2f(m[qt] - mn);  // 2^-inf = 0 while nothing was seen
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float pv = __builtin_amdgcn_exp2f(fmaf(sc[qt][tt][r], scale2, -mn));
+              rs += pv;
+              pop[qt][tt * 4 + r] = (bf16)pv;
+            }
+          m[qt] = mn;
+        }
+        rs += __shfl_xor(rs, 16, WAVE);
+        rs += __shfl_xor(rs, 32, WAVE);
+        l[qt] = l[qt] * alpha[qt] + rs;
+        rescale = rescale || alpha[qt] != 1.f;
+      }
+      // the accumulated output is rescaled only when some query's maximum moved (rare once the
+      // first keys have been seen)
+      if (__any(rescale)) {
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha[qt];
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        bf16x8_t vop;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const bf16x4_t v4 = *reinterpret_cast<const bf16x4_t*>(&lds_v[buf][tt][(dt * 16 + col) * 16 + 4 * grp]);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
+        }
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt], o[qt][dt], 0, 0, 0);
       }
     }
-    if (more) cur = nxt;
+    if (more) stash(buf ^ 1);
+    __syncthreads();
   }
 
 #pragma unroll
@@ -573,7 +672,7 @@ extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const vo
   if (num_tiles <= 0) return AS_OK;
   if (H <= 0 || KV <= 0 || H % KV || bs <= 0 || table_width <= 0) return AS_BAD_SHAPE;
   const int G = H / KV;
-  if (D % 32 || D <= 0 || D > 256 || bs % 16) return AS_BAD_SHAPE;
+  if (D % 32 || D <= 0 || D > 224 || bs % 16) return AS_BAD_SHAPE;  // wider heads: tiles exceed LDS
   dim3 grid(num_tiles, KV, (2 * G + 3) / 4);
 #define LAUNCH(DCV)                                                                                    \
   attn_prefill_mfma_kernel<DCV><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,       \
@@ -586,8 +685,7 @@ extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const vo
     case 4: LAUNCH(4); break;
     case 5: LAUNCH(5); break;
     case 6: LAUNCH(6); break;
-    case 7: LAUNCH(7); break;
-    default: LAUNCH(8); break;
+    default: LAUNCH(7); break;
   }
 #undef LAUNCH
   return launch_status();

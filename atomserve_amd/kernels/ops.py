@@ -189,9 +189,12 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
+PREFILL_MAX_HEAD_DIM = 224  # the staged key and value tiles of wider heads do not fit in LDS
+
+
 def attn_prefill_supported(dtype, head_dim: int, block_size: int) -> bool:
     """Whether `attn_prefill` takes this case; if not, the rows go through `attn_single_query`."""
-    return dtype == BF16 and head_dim % 32 == 0 and head_dim <= 256 and block_size % 16 == 0
+    return dtype == BF16 and head_dim % 32 == 0 and head_dim <= PREFILL_MAX_HEAD_DIM and block_size % 16 == 0
 
 
 def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context) -> None:
