@@ -143,3 +143,32 @@ def test_greedy_generation_through_the_entry_point(setup, dtype):
                 ref = plain.logits(raw, weights, seq)[-1]
                 assert ref[t] >= ref.max() - TOL["bfloat16"] * max(1.0, float(ref.abs().max())) * 2
                 seq.append(t)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_layer_sizes(dtype, tmp_path_factory):
+    """Two layers of Qwen3-8B's sizes (hidden 4096, 32/8 heads of 128, intermediate 12288) with a
+    smaller vocabulary: the kernels at the sizes they serve, whole, in portions and decoded."""
+    raw = {**TINY_B_LIKE_8B}
+    weights = plain_random_weights(raw, seed=77, std=0.02, gain_std=0.1)
+    path = write_model_dir(str(tmp_path_factory.mktemp("real")), raw, weights, torch.bfloat16)
+    ids = rc.random_ids(raw["vocab_size"], 150, seed=9)
+    cache = {"a": plain.logits(raw, weights, ids, dtype=torch.float32).float()}
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ids[:70], "want": list(range(0, 70, 7))}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": ids[70:75], "want": [0, 4]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": ids[75:140], "want": [0, 64]}], "end": []}]  # fmt: skip
+    steps += [{"step": 3 + i, "entries": [{"id": "a", "tokens": [ids[140 + i]], "want": [0]}], "end": []} for i in range(10)]
+    replay = make_replay(path, dtype, 192)
+    worst, scale, rows = rc.run_and_compare(replay, steps, {"a": ids}, raw, weights, cache)
+    assert rows == 24
+    # the plain side runs in float32 here (the float64 copy of these weights would not be worth its memory)
+    tol = {"float32": 1e-4, "bfloat16": TOL["bfloat16"]}[dtype]
+    assert worst <= tol * max(scale, 1.0), f"{dtype}: |difference| {worst:.3e} against |logits| {scale:.3e}"
+
+
+TINY_B_LIKE_8B = {
+    "architectures": ["Qwen3ForCausalLM"], "vocab_size": 20000, "hidden_size": 4096, "intermediate_size": 12288,
+    "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "tie_word_embeddings": False, "max_position_embeddings": 4096,
+    "hidden_act": "silu",
+}  # fmt: skip
