@@ -120,43 +120,73 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(const b
 #pragma unroll
   for (int s = 0; s < S; ++s) wrow[s] = w + (size_t)min(n0 + s * 16 + lr, N - 1) * K;
   const bf16* arow[MT];
-  bool aval[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + lr;
-    aval[mt] = m < M;
-    arow[mt] = a + (size_t)min(m, M - 1) * K;
-  }
+  for (int mt = 0; mt < MT; ++mt) arow[mt] = a + (size_t)min(mt * 16 + lr, M - 1) * K;
   floatx4 acc[S][MT];
 #pragma unroll
   for (int s = 0; s < S; ++s)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[s][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 2
-  for (int st = st0; st < st1; ++st) {
-    const int k = st * 64 + lg * 16;
+  // Main loop: whole 64-wide steps, four at a time, every load unconditional (rows beyond M or
+  // N were clamped to valid ones above; their results are never stored), so that sixteen or
+  // more 16-byte loads per lane are in flight before the first MFMA waits for data.
+  const int full_steps = K >> 6;
+  const int st_full = min(st1, full_steps);
+  int st = st0;
+#define SK_LOAD(U, STEP)                                                                     \
+  {                                                                                          \
+    const int k = (STEP) * 64 + lg * 16;                                                     \
+    _Pragma("unroll") for (int s = 0; s < S; ++s) {                                          \
+      wv[U][s][0] = *reinterpret_cast<const bf16x8*>(wrow[s] + k);                           \
+      wv[U][s][1] = *reinterpret_cast<const bf16x8*>(wrow[s] + k + 8);                       \
+    }                                                                                        \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                      \
+      av[U][mt][0] = *reinterpret_cast<const bf16x8*>(arow[mt] + k);                         \
+      av[U][mt][1] = *reinterpret_cast<const bf16x8*>(arow[mt] + k + 8);                     \
+    }                                                                                        \
+  }
+#define SK_MATH(U)                                                                                        \
+  _Pragma("unroll") for (int s = 0; s < S; ++s) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {       \
+    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[U][s][0], av[U][mt][0], acc[s][mt], 0, 0, 0); \
+    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[U][s][1], av[U][mt][1], acc[s][mt], 0, 0, 0); \
+  }
+#ifdef SK_UN_OVERRIDE
+  constexpr int UN = SK_UN_OVERRIDE;
+#else
+  constexpr int UN = (S * MT >= 4) ? 2 : 4;  // steps in flight; fewer when a step already holds many registers
+#endif
+  for (; st + UN <= st_full; st += UN) {
+    bf16x8 wv[UN][S][2], av[UN][MT][2];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) SK_LOAD(u, st + u)
+#pragma unroll
+    for (int u = 0; u < UN; ++u) SK_MATH(u)
+  }
+  for (; st < st_full; ++st) {
+    bf16x8 wv[1][S][2], av[1][MT][2];
+    SK_LOAD(0, st)
+    SK_MATH(0)
+  }
+#undef SK_LOAD
+  if (st0 <= full_steps && st1 > full_steps && (K & 63)) {  // the wave owning the last, partial step: chunks of 8 beyond K count as zeros
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int k = full_steps * 64 + lg * 16;
     const bool v0 = k + 8 <= K, v1 = k + 16 <= K;
-    bf16x8 wv[S][2], av[MT][2];
+    bf16x8 wv[1][S][2], av[1][MT][2];
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-      wv[s][0] = v0 ? *reinterpret_cast<const bf16x8*>(wrow[s] + k) : zero;
-      wv[s][1] = v1 ? *reinterpret_cast<const bf16x8*>(wrow[s] + k + 8) : zero;
+      wv[0][s][0] = v0 ? *reinterpret_cast<const bf16x8*>(wrow[s] + k) : zero;
+      wv[0][s][1] = v1 ? *reinterpret_cast<const bf16x8*>(wrow[s] + k + 8) : zero;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      av[mt][0] = (v0 && aval[mt]) ? *reinterpret_cast<const bf16x8*>(arow[mt] + k) : zero;
-      av[mt][1] = (v1 && aval[mt]) ? *reinterpret_cast<const bf16x8*>(arow[mt] + k + 8) : zero;
+      av[0][mt][0] = v0 ? *reinterpret_cast<const bf16x8*>(arow[mt] + k) : zero;
+      av[0][mt][1] = v1 ? *reinterpret_cast<const bf16x8*>(arow[mt] + k + 8) : zero;
     }
-#pragma unroll
-    for (int s = 0; s < S; ++s)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[s][0], av[mt][0], acc[s][mt], 0, 0, 0);
-        acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[s][1], av[mt][1], acc[s][mt], 0, 0, 0);
-      }
+    SK_MATH(0)
   }
+#undef SK_MATH
 
 #pragma unroll
   for (int s = 0; s < S; ++s)
@@ -187,6 +217,74 @@ static int launch_skinny(const void* a, const void* w, void* out, int out_dtype,
   return launch_status();
 }
 
+// The same product for up to 16 rows when K == 64 * WAVES * NST exactly: persistent
+// workgroups.  Each wave keeps its slice of the activations in registers for the whole
+// kernel and walks over strips of 16 weight rows (strip = blockIdx.x, + gridDim.x, ...), so
+// the activations are read once per workgroup instead of once per strip, no workgroup is
+// launched or retired while the weights stream, and all workgroups advance through memory
+// side by side.
+template <int NST, int WAVES, typename OutT>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_persistent_kernel(const bf16* __restrict__ a,
+                                                                                const bf16* __restrict__ w,
+                                                                                OutT* __restrict__ out, int M, int N,
+                                                                                int K, int nstrips) {
+  __shared__ floatx4 red[WAVES * 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int kbase = wave * NST * 64 + lg * 16;  // this lane's first k; step u adds 64 u
+  bf16x8 av[NST][2];
+  {
+    const bf16* arow = a + (size_t)min(lr, M - 1) * K + kbase;
+#pragma unroll
+    for (int u = 0; u < NST; ++u) {
+      av[u][0] = *reinterpret_cast<const bf16x8*>(arow + u * 64);
+      av[u][1] = *reinterpret_cast<const bf16x8*>(arow + u * 64 + 8);
+    }
+  }
+  for (int strip = blockIdx.x; strip < nstrips; strip += gridDim.x) {
+    const int n0 = strip * 16;
+    const bf16* wrow = w + (size_t)min(n0 + lr, N - 1) * K + kbase;
+    bf16x8 wv[NST][2];
+#pragma unroll
+    for (int u = 0; u < NST; ++u) {
+      wv[u][0] = *reinterpret_cast<const bf16x8*>(wrow + u * 64);
+      wv[u][1] = *reinterpret_cast<const bf16x8*>(wrow + u * 64 + 8);
+    }
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < NST; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u][0], av[u][0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u][1], av[u][1], acc, 0, 0, 0);
+    }
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+      floatx4 sum = red[lane];
+#pragma unroll
+      for (int x = 1; x < WAVES; ++x) sum += red[x * 64 + lane];
+      const int m = lr, n = n0 + 4 * lg;
+      if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
+    }
+    __syncthreads();
+  }
+}
+
+template <int NST, int WAVES>
+static int launch_persistent(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
+                             hipStream_t stream) {
+  const int nstrips = (N + 15) / 16;
+  const int blocks = nstrips < 512 ? nstrips : 512;  // two workgroups per compute unit
+  if (out_dtype == DT_BF16)
+    gemm_bf16_skinny_persistent_kernel<NST, WAVES, bf16><<<blocks, WAVES * 64, 0, stream>>>(
+        (const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, nstrips);
+  else if (out_dtype == DT_F32)
+    gemm_bf16_skinny_persistent_kernel<NST, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>(
+        (const bf16*)a, (const bf16*)w, (float*)out, M, N, K, nstrips);
+  else
+    return AS_BAD_DTYPE;
+  return launch_status();
+}
+
 // strips: rows of w per workgroup / 16 (1, 2 or 4); 0 lets the kernel choose.
 // Few strips (a small N) get 16 waves per workgroup, so that K is split further and the
 // GPU still has enough loads in flight.
@@ -195,8 +293,17 @@ extern "C" int as_gemm_bf16_skinny(const void* a, const void* w, void* out, int 
   if (M <= 0) return AS_OK;
   if (M > 64 || N <= 0 || K <= 0 || (K & 7)) return AS_BAD_SHAPE;
   const int MT = (M + 15) / 16;
+  if (MT == 1 && ((strips == 0 && M > 8) || strips == -1)) {  // measured: pays from 9 rows on
+    // persistent kernel when K splits exactly over the waves; many strips -> 8 waves, few -> 16
+    const bool wide = (N + 15) / 16 < 512;
+    if (!wide && K == 64 * 8 * 8) return launch_persistent<8, 8>(a, w, out, out_dtype, M, N, K, stream);
+    if (!wide && K == 64 * 8 * 4) return launch_persistent<4, 8>(a, w, out, out_dtype, M, N, K, stream);
+    if (wide && K == 64 * 16 * 4) return launch_persistent<4, 16>(a, w, out, out_dtype, M, N, K, stream);
+    if (wide && K == 64 * 16 * 8) return launch_persistent<8, 16>(a, w, out, out_dtype, M, N, K, stream);
+    if (strips == -1) return AS_BAD_SHAPE;
+  }
   int S = strips;
-  if (S == 0) S = (MT > 2) ? 1 : (N >= 65536 ? 4 : (N >= 6144 ? 2 : 1));
+  if (S == 0) S = 1;  // measured best at every size of interest; more strips only cost registers
   if (MT > 2 && S > 1) S = 1;  // keeps the partial sums within LDS
   const bool wide = (N / (16 * S)) < 512 && MT <= 2 && S == 1;
 #define CASE(SV, MTV)                                                                               \

@@ -184,7 +184,8 @@ def test_gemm_fp32_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one[0], full[i])
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (64, 4096, 1024), (300, 257, 192), (5, 2000, 4096)])
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (64, 4096, 1024), (300, 257, 192), (5, 2000, 4096),
+                                   (16, 4096, 4096), (12, 8200, 4096), (9, 16000, 2048), (3, 40, 200), (16, 24, 8)])
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(8)
     a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
