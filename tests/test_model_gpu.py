@@ -172,3 +172,19 @@ TINY_B_LIKE_8B = {
     "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "tie_word_embeddings": False, "max_position_embeddings": 4096,
     "hidden_act": "silu",
 }  # fmt: skip
+
+
+def test_a_folder_stored_in_32_bit_served_in_bfloat16(tmp_path):
+    """Matrices follow the serving dtype; gains stored in 32-bit stay 32-bit and the kernels take
+    them so."""
+    raw = TINY["B"]
+    weights = plain_random_weights(raw, seed=91, std=0.2, gain_std=0.2)
+    path = write_model_dir(str(tmp_path / "m"), raw, weights, torch.float32)
+    ids = rc.random_ids(raw["vocab_size"], 90, seed=6)
+    replay = make_replay(path, "bfloat16", 128)
+    assert replay.model.blocks[0].mixer.q_norm_weight.dtype == torch.float32
+    assert replay.model.blocks[0].mixer.qkv_weight.dtype == torch.bfloat16
+    steps = rc.portions("a", ids, sizes=(40, 3, 1, 1, 30, 15))
+    worst, scale, rows = rc.run_and_compare(replay, steps, {"a": ids}, raw, weights, {})
+    assert rows == 90
+    check(worst, scale, "bfloat16")
