@@ -135,6 +135,13 @@ def test_greedy_generation_through_the_entry_point(setup, dtype):
         tight = engine(num_blocks=sum(-(-len(p) // bs) for p in prompts), max_model_len=64)
         assert tight.generate(prompts, params) == together
         assert tight.stats()["preemptions"] > 0 and tight.stats()["kv_blocks_used"] == 0
+        # the same prompts again on one engine: their full pages are found in the prefix cache
+        warm = engine()
+        assert warm.generate(prompts, params) == together
+        before = warm.stats()["cached_prompt_tokens"]
+        assert warm.generate(prompts, params) == together
+        assert warm.stats()["cached_prompt_tokens"] >= before + (33 // bs) * bs
+        assert engine(enable_prefix_caching=False).generate(prompts, params) == together
     else:
         # bf16 may flip near-ties; every token must still be (nearly) the best under the plain logits
         for p, out in zip(prompts, together):
@@ -188,3 +195,26 @@ def test_a_folder_stored_in_32_bit_served_in_bfloat16(tmp_path):
     worst, scale, rows = rc.run_and_compare(replay, steps, {"a": ids}, raw, weights, {})
     assert rows == 90
     check(worst, scale, "bfloat16")
+
+
+def test_command_line_generates(setup, capsys):
+    """`atomserve <folder> --prompt-ids ...` end to end: greedy tokens equal the plain model's."""
+    import json as js
+
+    from atomserve_amd.engine.cli import main
+
+    name, raw, weights, path, _ = setup
+    prompts = [[3, 14, 15, 9, 2], [6, 5]]
+    argv = [path, "--dtype", "fp32", "--temperature", "0", "--max-tokens", "5", "--ignore-eos", "--kv-mem-gb", "0.01",
+            "--max-num-seqs", "4", "--max-batched-tokens", "16"]  # fmt: skip
+    for p in prompts:
+        argv += ["--prompt-ids", ",".join(map(str, p))]
+    assert main(argv) == 0
+    lines = [js.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert [r["output_ids"] for r in lines] == [plain.greedy(raw, weights, p, 5) for p in prompts]
+    assert all(r["finish_reason"] == "length" for r in lines)
+    # and with weights drawn from a seed instead of read from the folder
+    assert main([path, "--random-weights", "3", "--temperature", "0.7", "--seed", "1", "--max-tokens", "4", "--prompt-ids", "1 2 3",
+                 "--kv-mem-gb", "0.01", "--max-num-seqs", "4", "--max-batched-tokens", "16"]) == 0  # fmt: skip
+    out = [js.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert len(out) == 1 and len(out[0]["output_ids"]) <= 4
