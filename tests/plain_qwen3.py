@@ -85,7 +85,8 @@ def swiglu(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: to
 
 
 def attention_layer(x, w, prefix, cfg, positions):  # positions are absolute
-    """Projection, per-head RMSNorm of q and k (same eps as the layer norms, before the
+    """(cfg["window"], if present, limits the keys a query sees; Qwen3 has none.)
+    Projection, per-head RMSNorm of q and k (same eps as the layer norms, before the
     rotation, v untouched), rotation, attention, output projection
     (reference atomserve/model.py:317-336)."""
     T = x.shape[0]
@@ -97,7 +98,7 @@ def attention_layer(x, w, prefix, cfg, positions):  # positions are absolute
     q = rms_norm(q, w[prefix + "self_attn.q_norm.weight"], eps)
     k = rms_norm(k, w[prefix + "self_attn.k_norm.weight"], eps)
     q, k = rope(q, positions, theta), rope(k, positions, theta)
-    o = causal_attention(q, k, v, positions, k_positions=positions)
+    o = causal_attention(q, k, v, positions, window=cfg.get("window", 0), k_positions=positions)
     return o.reshape(T, H * D) @ w[prefix + "self_attn.o_proj.weight"].T
 
 

@@ -131,7 +131,8 @@ def build_engine(arch, raw, weights, dtype, device=DEV, **engine):
 
 
 def step_rows(engine, caches, entries):
-    """entries: (name, tokens, want) -> logits; requests keep their pages and slots in `caches`."""
+    """entries: (name, tokens, want) -> logits; requests keep their pages and slots in `caches`;
+    after the step, pages that a window has passed are given back."""
     from atomserve_amd.engine.batch import Row
 
     m = engine.scheduler.manager
@@ -141,7 +142,10 @@ def step_rows(engine, caches, entries):
         assert m.reserve(rc, done, len(tokens))
         rows.append(Row(tokens, done, rc.tables, want, rc.state_slot))
         caches[name][1] += len(tokens)
-    return engine.runner.step(rows).float().cpu()
+    logits = engine.runner.step(rows).float().cpu()
+    for name, _, _ in entries:
+        m.release_behind_window(*caches[name])
+    return logits
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -244,6 +248,79 @@ def test_a_layer_runs_twice_and_reads_the_cache_of_its_first_run(dtype, device=D
     got += [step_rows(engine, caches, [("a", [ids[i]], [0])]) for i in range(21, 30)]
     got.append(step_rows(engine, caches, [("a", ids[30:], list(range(10)))]))
     assert (torch.cat(got) - ref).abs().max() <= tol * max(1.0, ref.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layers_with_a_window_have_pages_of_their_own_and_give_them_back(dtype, device=DEV):
+    """Odd layers see the last 24 keys only: two cache groups, each with its pool and tables.
+    The windowed group's pool is smaller than one request's length, so it only works because
+    pages behind the window return to the pool and are handed out again, to the same and to
+    the other request; what they held before must never show."""
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+
+    qwen = architecture_for(TINY_B)
+    window = 24
+
+    def build_plan(c):
+        plan = qwen.build_plan(c)
+        layers = tuple(dataclasses.replace(layer, mixer=dataclasses.replace(layer.mixer, window=window)) if i % 2 else layer
+                       for i, layer in enumerate(plan.layers))  # fmt: skip
+        return dataclasses.replace(plan, layers=layers)
+
+    arch = register_architecture(
+        Architecture("WindowedForCausalLM", qwen.parse_config, build_plan, qwen.checkpoint_map, qwen.checkpoint_shapes), replace=True
+    )
+    raw = {**TINY_B, "architectures": ["WindowedForCausalLM"], "num_hidden_layers": 4}
+    w = plain_random_weights(raw, seed=8, std=0.2, gain_std=0.2)
+    engine = build_engine(arch, raw, w, dtype, device, num_blocks=24, max_model_len=384)
+    m = engine.scheduler.manager
+    assert [(g.window, g.cache_ids) for g in m.paged_groups] == [(0, [0, 2]), (window, [1, 3])]
+    a = torch.randint(0, 1000, (170,), generator=torch.Generator().manual_seed(4)).tolist()
+    b = torch.randint(0, 1000, (150,), generator=torch.Generator().manual_seed(5)).tolist()
+
+    def reference(ids):
+        cfg = plain.normalise_config(raw)
+        wd = {k: v.double() for k, v in w.items()}
+        pos = torch.arange(len(ids))
+        x = plain.embed(wd["model.embed_tokens.weight"], torch.as_tensor(ids))
+        for i in range(4):
+            p = f"model.layers.{i}."
+            h = plain.rms_norm(x, wd[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+            x = x + plain.attention_layer(h, wd, p, {**cfg, "window": window if i % 2 else 0}, pos)
+            h = plain.rms_norm(x, wd[p + "post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+            x = x + plain.swiglu(h, wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"], wd[p + "mlp.down_proj.weight"])
+        x = plain.rms_norm(x, wd["model.norm.weight"], cfg["rms_norm_eps"])
+        return (x @ wd["lm_head.weight"].T).float()
+
+    ref = {"a": reference(a), "b": reference(b)}
+    caches, got, at = {}, {"a": [], "b": []}, {"a": 0, "b": 0}
+    held_most = 0
+    plan = [("a", 50), ("b", 3), ("a", 1), ("b", 70), ("a", 1), ("a", 30), ("b", 1), ("a", 2), ("b", 40), ("a", 66), ("b", 36), ("a", 20)]
+    ids = {"a": a, "b": b}
+    i = 0
+    while i < len(plan):
+        entries = []
+        for name, n in plan[i : i + 2] if plan[i][0] != plan[min(i + 1, len(plan) - 1)][0] else plan[i : i + 1]:
+            entries.append((name, ids[name][at[name] : at[name] + n], list(range(n))))
+            at[name] += n
+        i += len(entries)
+        logits = step_rows(engine, caches, entries)
+        k = 0
+        for name, tokens, _ in entries:
+            got[name].append(logits[k : k + len(tokens)])
+            k += len(tokens)
+        windowed = m.paged_groups[1].allocator
+        held_most = max(held_most, windowed.num_pages - windowed.num_free)
+    assert at == {"a": 170, "b": 150}
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    for name in "ab":
+        assert (torch.cat(got[name]) - ref[name]).abs().max() <= tol * max(1.0, ref[name].abs().max()), name
+    # 320 tokens went through the windowed layers on at most a handful of pages at a time
+    assert held_most <= 2 * (-(-(window + 70) // 16) + 1)
+    assert sum(1 for p in caches["a"][0].tables[1] if p == -1) >= 8  # given back as the window moved on
+    for rc, _ in caches.values():
+        m.release(rc)
+    assert all(g.allocator.num_free == 24 for g in m.paged_groups)
 
 
 # ---- each part alone ------------------------------------------------------------------------
