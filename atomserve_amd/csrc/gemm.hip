@@ -217,89 +217,187 @@ static int launch_skinny(const void* a, const void* w, void* out, int out_dtype,
   return launch_status();
 }
 
-// The same product for up to 16 rows when K == 64 * WAVES * NST exactly: persistent
-// workgroups.  Each wave keeps its slice of the activations in registers for the whole
-// kernel and walks over strips of 16 weight rows (strip = blockIdx.x, + gridDim.x, ...), so
-// the activations are read once per workgroup instead of once per strip, no workgroup is
-// launched or retired while the weights stream, and all workgroups advance through memory
-// side by side.
-template <int NST, int WAVES, typename OutT>
-__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_persistent_kernel(const bf16* __restrict__ a,
-                                                                                const bf16* __restrict__ w,
-                                                                                OutT* __restrict__ out, int M, int N,
-                                                                                int K, int nstrips) {
-  __shared__ floatx4 red[WAVES * 64];
+// The same product for up to 16 rows and K <= 64 * PIPE_WAVES * NST: persistent workgroups,
+// one per compute unit.  Measured on the streaming kernel above: re-reading the activations
+// for every strip costs as much as a fifth of the weights' own traffic.  Here each wave keeps
+// its K-slice of the activations in registers for the whole kernel and walks over strips of
+// 16 weight rows (strip = blockIdx.x, + gridDim.x, ...).  A strip's weights sit in two
+// register buffers (first and second half of the wave's slice); as soon as a half has gone
+// through the matrix cores, the same half of the NEXT strip is requested, so loads stay in
+// flight while the partial sums of the waves meet in LDS.  The LDS buffer alternates between
+// strips, which leaves one barrier per strip; the wave that adds and stores rotates.
+// Chunks of 8 beyond K count as zeros (MASKED), so any K % 8 == 0 up to the limit is taken.
+//
+// GATED: w holds N gate rows followed by N up rows, and out[m, n] = silu(gate) * up with both
+// sums rounded to OutT first, which is what the plain product followed by the activation
+// kernel gives.  A workgroup then walks over pairs of strips (gate rows, then the up rows of
+// the same outputs); the wave whose turn it is keeps the gate sums until the up sums arrive.
+constexpr int PIPE_WAVES = 8;
+constexpr int PIPE_MAX_NST = 12;
+
+template <typename OutT> __device__ __forceinline__ float rounded(float v);
+template <> __device__ __forceinline__ float rounded<float>(float v) { return v; }
+template <> __device__ __forceinline__ float rounded<bf16>(float v) { return (float)(bf16)v; }
+
+template <int NST, bool MASKED, bool GATED, typename OutT>
+__global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(const bf16* __restrict__ a,
+                                                                               const bf16* __restrict__ w,
+                                                                               OutT* __restrict__ out, int M, int N,
+                                                                               int K, int nstrips) {
+  static_assert(NST % 2 == 0, "a wave's slice is handled in two halves");
+  constexpr int H = NST / 2;
+  __shared__ floatx4 red[2][PIPE_WAVES * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
   const int kbase = wave * NST * 64 + lg * 16;  // this lane's first k; step u adds 64 u
+  // A unit of work is 16 rows of w: `strip` counts strips of outputs, `up` says which half
+  // of a gated w the rows come from.
+  int strip = blockIdx.x;
+  bool up = false;
+  if (strip >= nstrips) return;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#define PIPE_VALID(U, HALF) (!MASKED || kbase + (U) * 64 + (HALF) * 8 + 8 <= K)
+#define PIPE_LOAD(BUF, ROW, OFF)                                                                              \
+  _Pragma("unroll") for (int u = 0; u < H; ++u) {                                                             \
+    BUF[u][0] = PIPE_VALID((OFF) + u, 0) ? *reinterpret_cast<const bf16x8*>(ROW + ((OFF) + u) * 64) : zero;   \
+    BUF[u][1] = PIPE_VALID((OFF) + u, 1) ? *reinterpret_cast<const bf16x8*>(ROW + ((OFF) + u) * 64 + 8) : zero; \
+  }
+#define PIPE_MATH(BUF, OFF)                                                                   \
+  _Pragma("unroll") for (int u = 0; u < H; ++u) {                                             \
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][0], av[(OFF) + u][0], acc, 0, 0, 0); \
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][1], av[(OFF) + u][1], acc, 0, 0, 0); \
+  }
+#define PIPE_ROWS(STRIP, UP) (w + ((size_t)min((STRIP) * 16 + lr, N - 1) + ((UP) ? (size_t)N : 0)) * K + kbase)
+  bf16x8 w0[H][2], w1[H][2];
+  const bf16* wrow = PIPE_ROWS(strip, false);
+  PIPE_LOAD(w0, wrow, 0)
+  PIPE_LOAD(w1, wrow, H)
   bf16x8 av[NST][2];
   {
     const bf16* arow = a + (size_t)min(lr, M - 1) * K + kbase;
 #pragma unroll
     for (int u = 0; u < NST; ++u) {
-      av[u][0] = *reinterpret_cast<const bf16x8*>(arow + u * 64);
-      av[u][1] = *reinterpret_cast<const bf16x8*>(arow + u * 64 + 8);
+      av[u][0] = PIPE_VALID(u, 0) ? *reinterpret_cast<const bf16x8*>(arow + u * 64) : zero;
+      av[u][1] = PIPE_VALID(u, 1) ? *reinterpret_cast<const bf16x8*>(arow + u * 64 + 8) : zero;
     }
   }
-  for (int strip = blockIdx.x; strip < nstrips; strip += gridDim.x) {
-    const int n0 = strip * 16;
-    const bf16* wrow = w + (size_t)min(n0 + lr, N - 1) * K + kbase;
-    bf16x8 wv[NST][2];
-#pragma unroll
-    for (int u = 0; u < NST; ++u) {
-      wv[u][0] = *reinterpret_cast<const bf16x8*>(wrow + u * 64);
-      wv[u][1] = *reinterpret_cast<const bf16x8*>(wrow + u * 64 + 8);
-    }
+  int buf = 0, turn = 0;
+  floatx4 gate = {0.f, 0.f, 0.f, 0.f};
+  for (;;) {
+    const bool next_up = GATED && !up;
+    const int next = next_up ? strip : strip + gridDim.x;
+    const bool more = next < nstrips;
+    const bf16* nrow = PIPE_ROWS(next, next_up);
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int u = 0; u < NST; ++u) {
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u][0], av[u][0], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u][1], av[u][1], acc, 0, 0, 0);
-    }
-    red[wave * 64 + lane] = acc;
+    PIPE_MATH(w0, 0)
+    if (more) { PIPE_LOAD(w0, nrow, 0) }
+    PIPE_MATH(w1, H)
+    if (more) { PIPE_LOAD(w1, nrow, H) }
+    red[buf][wave * 64 + lane] = acc;
     __syncthreads();
-    if (wave == 0) {
-      floatx4 sum = red[lane];
+    if (wave == turn) {  // sums in the order of the waves, whichever wave adds them
+      floatx4 sum = red[buf][lane];
 #pragma unroll
-      for (int x = 1; x < WAVES; ++x) sum += red[x * 64 + lane];
-      const int m = lr, n = n0 + 4 * lg;
-      if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
+      for (int x = 1; x < PIPE_WAVES; ++x) sum += red[buf][x * 64 + lane];
+      if (GATED && !up) {
+        gate = sum;
+      } else {
+        if (GATED) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float g = rounded<OutT>(gate[r]);
+            sum[r] = g / (1.0f + expf(-g)) * rounded<OutT>(sum[r]);
+          }
+        }
+        const int m = lr, n = strip * 16 + 4 * lg;
+        if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
+      }
     }
-    __syncthreads();
+    if (!more) break;
+    // The next strip writes the other LDS buffer, and its barrier comes before anyone writes
+    // this one again; by then the adding wave has passed that barrier, so it has read this one.
+    buf ^= 1;
+    if (!next_up) turn = (turn + 1 == PIPE_WAVES) ? 0 : turn + 1;
+    strip = next;
+    up = next_up;
   }
+#undef PIPE_ROWS
+#undef PIPE_VALID
+#undef PIPE_LOAD
+#undef PIPE_MATH
 }
 
-template <int NST, int WAVES>
-static int launch_persistent(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
-                             hipStream_t stream) {
+static int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <int NST, bool GATED>
+static int launch_pipe(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
+                       hipStream_t stream) {
   const int nstrips = (N + 15) / 16;
-  const int blocks = nstrips < 512 ? nstrips : 512;  // two workgroups per compute unit
-  if (out_dtype == DT_BF16)
-    gemm_bf16_skinny_persistent_kernel<NST, WAVES, bf16><<<blocks, WAVES * 64, 0, stream>>>(
-        (const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, nstrips);
-  else if (out_dtype == DT_F32)
-    gemm_bf16_skinny_persistent_kernel<NST, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>(
-        (const bf16*)a, (const bf16*)w, (float*)out, M, N, K, nstrips);
-  else
+  const int blocks = min(nstrips, compute_units());
+  const bool exact = K == 64 * PIPE_WAVES * NST;
+#define PIPE_GO(MASKED, OutT)                                                                        \
+  gemm_bf16_skinny_pipe_kernel<NST, MASKED, GATED, OutT><<<blocks, PIPE_WAVES * 64, 0, stream>>>(    \
+      (const bf16*)a, (const bf16*)w, (OutT*)out, M, N, K, nstrips)
+  if (out_dtype == DT_BF16) {
+    if (exact) PIPE_GO(false, bf16); else PIPE_GO(true, bf16);
+  } else if (out_dtype == DT_F32) {
+    if (exact) PIPE_GO(false, float); else PIPE_GO(true, float);
+  } else {
     return AS_BAD_DTYPE;
+  }
+#undef PIPE_GO
   return launch_status();
 }
 
-// strips: rows of w per workgroup / 16 (1, 2 or 4); 0 lets the kernel choose.
-// Few strips (a small N) get 16 waves per workgroup, so that K is split further and the
-// GPU still has enough loads in flight.
+template <bool GATED>
+static int dispatch_pipe(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
+                         hipStream_t stream) {
+  switch (2 * ((K + 128 * PIPE_WAVES - 1) / (128 * PIPE_WAVES))) {
+    case 2: return launch_pipe<2, GATED>(a, w, out, out_dtype, M, N, K, stream);
+    case 4: return launch_pipe<4, GATED>(a, w, out, out_dtype, M, N, K, stream);
+    case 6: return launch_pipe<6, GATED>(a, w, out, out_dtype, M, N, K, stream);
+    case 8: return launch_pipe<8, GATED>(a, w, out, out_dtype, M, N, K, stream);
+    case 10: return launch_pipe<10, GATED>(a, w, out, out_dtype, M, N, K, stream);
+    case 12: return launch_pipe<12, GATED>(a, w, out, out_dtype, M, N, K, stream);
+  }
+  return AS_BAD_SHAPE;
+}
+
+// Whether the persistent kernel takes a product of these sizes.
+static bool pipe_fits(int M, int K) { return M <= 16 && K <= 64 * PIPE_WAVES * PIPE_MAX_NST; }
+
+// out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for w[2N, K], both products rounded to the
+// output type before the activation.  Only sizes of the persistent kernel; AS_BAD_SHAPE
+// otherwise, and the caller runs the product and the activation kernel instead.
+extern "C" int as_gemm_bf16_gated(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
+                                  hipStream_t stream) {
+  if (M <= 0) return AS_OK;
+  if (N <= 0 || K <= 0 || (K & 7) || !pipe_fits(M, K)) return AS_BAD_SHAPE;
+  return dispatch_pipe<true>(a, w, out, out_dtype, M, N, K, stream);
+}
+
+// strips: rows of w per workgroup / 16 in the streaming kernel (1, 2 or 4); 0 lets this
+// function choose, which for up to 16 rows and a K that fits is the persistent kernel (-1
+// asks for that one and fails where it cannot run).  Few strips (a small N) get 16 waves
+// per workgroup in the streaming kernel, so that K is split further and the GPU still has
+// enough loads in flight.
 extern "C" int as_gemm_bf16_skinny(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
                                    int strips, hipStream_t stream) {
   if (M <= 0) return AS_OK;
   if (M > 64 || N <= 0 || K <= 0 || (K & 7)) return AS_BAD_SHAPE;
   const int MT = (M + 15) / 16;
-  if (MT == 1 && ((strips == 0 && M > 8) || strips == -1)) {  // measured: pays from 9 rows on
-    // persistent kernel when K splits exactly over the waves; many strips -> 8 waves, few -> 16
-    const bool wide = (N + 15) / 16 < 512;
-    if (!wide && K == 64 * 8 * 8) return launch_persistent<8, 8>(a, w, out, out_dtype, M, N, K, stream);
-    if (!wide && K == 64 * 8 * 4) return launch_persistent<4, 8>(a, w, out, out_dtype, M, N, K, stream);
-    if (wide && K == 64 * 16 * 4) return launch_persistent<4, 16>(a, w, out, out_dtype, M, N, K, stream);
-    if (wide && K == 64 * 16 * 8) return launch_persistent<8, 16>(a, w, out, out_dtype, M, N, K, stream);
+  if (strips == 0 || strips == -1) {
+    if (pipe_fits(M, K)) return dispatch_pipe<false>(a, w, out, out_dtype, M, N, K, stream);
     if (strips == -1) return AS_BAD_SHAPE;
   }
   int S = strips;

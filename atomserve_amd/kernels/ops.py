@@ -248,6 +248,28 @@ def gemm(a, w, out) -> None:
         out.copy_(torch.mm(a, w.t()))
 
 
+GATED_MAX_K = 6144  # the widest input the fused product-and-activation kernel keeps in registers
+
+
+def gemm_silu_mul(a, w, out) -> None:
+    """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for w[2 I, K]: the gate and up products and
+    the activation.  bf16 with few rows: one kernel, the products rounded to bf16 before the
+    activation exactly as the two-kernel path does; otherwise the product, then the activation."""
+    _check(a, "a", (F32, BF16), (None, None))
+    M, K = a.shape
+    _check(out, "out", a.dtype, (M, None))
+    inter = out.shape[1]
+    _check(w, "w", a.dtype, (2 * inter, K))
+    if M == 0:
+        return
+    if a.dtype == BF16 and M <= SKINNY_MAX_ROWS and K % 8 == 0 and K <= GATED_MAX_K:
+        call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, inter, K, _stream())
+        return
+    gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
+    gemm(a, w, gate_up)
+    silu_mul(gate_up, out)
+
+
 SAMPLE_MAX_TOP_K = 1024
 
 

@@ -23,10 +23,8 @@ class GatedMLP(FeedForward):
     def forward(self, h, step):
         s, env = self.spec, self.env
         T = h.shape[0]
-        gate_up = torch.empty((T, 2 * s.intermediate_size), dtype=env.dtype, device=h.device)
-        ops.gemm(h, self.gate_up_weight, gate_up)
         act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=h.device)
-        ops.silu_mul(gate_up, act)
+        ops.gemm_silu_mul(h, self.gate_up_weight, act)
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=h.device)
         ops.gemm(act, self.down_weight, y)
         return y

@@ -185,7 +185,9 @@ def test_gemm_fp32_rows_do_not_depend_on_the_batch(ops):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (64, 4096, 1024), (300, 257, 192), (5, 2000, 4096),
-                                   (16, 4096, 4096), (12, 8200, 4096), (9, 16000, 2048), (3, 40, 200), (16, 24, 8)])
+                                   (16, 4096, 4096), (12, 8200, 4096), (9, 16000, 2048), (3, 40, 200), (16, 24, 8),
+                                   (4, 1040, 5120), (7, 520, 6144), (2, 100, 2560), (11, 4100, 3072), (8, 512, 12288),
+                                   (13, 300, 6152), (17, 300, 4096)])  # fmt: skip
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(8)
     a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
@@ -196,6 +198,34 @@ def test_gemm_bf16(ops, M, N, K):
     out32 = torch.empty(M, N, dtype=F32, device=DEV)
     ops.gemm(a, w, out32)
     assert torch.allclose(out32, ref, atol=math.sqrt(K) * 2.0**-8, rtol=2.0**-7)
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 12288, 4096), (9, 700, 2048),
+                                   (3, 40, 200), (16, 24, 8), (4, 520, 5120), (7, 264, 6144), (8, 128, 12288),
+                                   (40, 300, 512)])  # fmt: skip
+def test_gemm_silu_mul_bf16(ops, M, I, K):
+    """Gate and up products with the activation in one kernel (few rows, an input that fits)
+    or as product then activation: the same numbers as the two kernels give, which are the plain
+    activation of the products rounded to bfloat16."""
+    torch.manual_seed(9)
+    a, w = torch.randn(M, K, device=DEV).to(BF16), (torch.randn(2 * I, K, device=DEV) / math.sqrt(K)).to(BF16)
+    out = torch.empty(M, I, dtype=BF16, device=DEV)
+    ops.gemm_silu_mul(a, w, out)
+    gate_up = torch.empty(M, 2 * I, dtype=BF16, device=DEV)
+    ops.gemm(a, w, gate_up)
+    two = torch.empty(M, I, dtype=BF16, device=DEV)
+    ops.silu_mul(gate_up, two)
+    assert torch.equal(out, two)
+    assert close_bf16(gate_up, pk.gemm(a, w), scale=1.0)
+    assert close_bf16(out, pk.silu_mul(gate_up))
+
+
+def test_gemm_silu_mul_fp32(ops):
+    torch.manual_seed(10)
+    a, w = torch.randn(5, 72, device=DEV), torch.randn(2 * 50, 72, device=DEV) / 8
+    out = torch.empty(5, 50, device=DEV)
+    ops.gemm_silu_mul(a, w, out)
+    assert torch.allclose(out, pk.silu_mul(pk.gemm(a, w)), atol=1e-5, rtol=1e-5)
 
 
 def paged_case(dtype, H, KV, D, bs, lens, seed=0, k_scale=4.0):
