@@ -439,29 +439,73 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 // token, count, block-table row, position of the first) for one kv head.  A wave owns 32
 // of those queries for one query head, as two MFMA column tiles of 16; the four waves of a
 // workgroup take heads of the same group (or the other half of the queries), so they all
-// need the same keys and values.  Those are brought into LDS once per workgroup, 32 keys
-// per step: a 16-key piece of a page is contiguous in memory both for keys and, thanks to
-// the transposed value pages, for values, so every thread copies 16 bytes.  The next step
-// is on its way from memory while the current one is computed (double-buffered LDS).
+// need the same keys and values.  Those come into LDS once per workgroup by loads that write
+// LDS directly (global_load_lds_dwordx4: no staging registers), into a ring of four stages
+// of 32 keys.  A round of the main loop computes 64 keys (two stages) while the copies of the
+// next 64 are in flight into the other two, and costs one barrier; 64 keys give a wave 64
+// independent MFMAs between its softmax reductions, which is what hides their latency.
+// Each wave copies one of a stage's four 16-key pieces (keys 0-15, keys 16-31, values 0-15,
+// values 16-31): such a piece of a page is contiguous in memory both for keys and, thanks
+// to the transposed value pages, for values.
+//
+// LDS layout of a piece, in 16-byte slots:
+//   keys:   slot (c * 16 + r) holds coordinates 8c .. 8c+7 of key row r, so the 64 lanes of
+//           an MFMA operand read (row = lane % 16, chunk = 4 step + lane / 16) touch 64
+//           consecutive slots: no bank conflicts, no padding, any head width;
+//   values: the page's own order [coordinate][16 keys].
+// A load instruction fills 64 consecutive slots (slot = first + lane); which 16 bytes of
+// memory a lane fetches is free, which is how the key layout comes about.
 // A query at position p sees keys lo..p by absolute position, wherever the row starts.
-#define PF_PAD 8  // bf16 elements of padding per key row in LDS: spreads the rows over the banks
+// Sums and maxima over the four lanes that share `lane % 16` (lane ^ 16, lane ^ 32) without a
+// trip through LDS: v_permlane16_swap / v_permlane32_swap exchange rows of 16 lanes between
+// two registers.  With both operands equal to x, the results hold (rows 0 0 2 2, rows 1 1 3 3)
+// and (rows 0 1 0 1, rows 2 3 2 3) of x.
+__device__ __forceinline__ float quad_rows_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+#define PF_STAGES 4
+// s_waitcnt that only constrains the vector-memory counter (vmcnt: bits 3:0 and 15:14)
+#define PF_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 template <int DC>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ tiles, const int* __restrict__ block_tables, int table_width,
-    bf16* __restrict__ out, int H, int KV, int bs, float scale, int window) {
+    bf16* __restrict__ out, int H, int KV, int bs, float scale, int window, int units_z, int pass) {
   constexpr int D = DC * 32, DT = DC * 2;
-  constexpr int KROW = D + PF_PAD;               // elements per key row in LDS
-  constexpr int KTILE = 16 * KROW, VTILE = D * 16;  // elements per 16-key tile
-  constexpr int CHUNKS = 2 * D;                  // 16-byte chunks per tile (keys or values)
-  constexpr int PER = (CHUNKS + 255) / 256;      // chunks per thread per tile
-  __shared__ __attribute__((aligned(16))) bf16 lds_k[2][2][KTILE];
-  __shared__ __attribute__((aligned(16))) bf16 lds_v[2][2][VTILE];
+  constexpr int PIECE = 64 * DC;  // 16-byte slots of a 16-key piece: 16 * D / 8
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* global_ptr_t;
+  __shared__ __attribute__((aligned(16))) u32x4_t lds[PF_STAGES][4][PIECE];  // [stage][K0 K1 V0 V1][slot]
 
   const int G = H / KV;
-  const int tile = blockIdx.x, kvh = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // Work items (tile, kv head, group of four waves) in the order of `tiles`, which the caller
+  // sorts by the number of keys seen, most first; blocks of `pass` items alternate direction.
+  // With one pass per round of workgroups that the GPU places (its compute units), a compute
+  // unit that received one of the longest items in one round receives one of the shortest of
+  // the next, so that causal prompts, whose items range from one step to hundreds, finish
+  // together.
+  const int per_tile = KV * units_z;
+  int item = blockIdx.x;
+  {
+    const int block = item / pass, first = block * pass;
+    const int size = min(pass, (int)gridDim.x - first);
+    if (block & 1) item = first + size - 1 - (item - first);
+  }
+  const int tile = item / per_tile, kvh = (item % per_tile) / units_z, bz = item % units_z;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, grp = lane >> 4;
   const int tok0 = tiles[4 * tile], count = tiles[4 * tile + 1], row = tiles[4 * tile + 2];
   const int pos0 = tiles[4 * tile + 3];
@@ -469,7 +513,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
 
   // the keys this workgroup walks: from the first key any of its waves sees to the last
   int wg_lo = 0x7fffffff, wg_last = -1;
-  for (int u = blockIdx.z * 4; u < blockIdx.z * 4 + 4 && u < 2 * G; ++u) {
+  for (int u = bz * 4; u < bz * 4 + 4 && u < 2 * G; ++u) {
     const int uq0 = (u / G) * 32;
     if (uq0 >= count) continue;
     wg_last = max(wg_last, pos0 + min(count, uq0 + 32) - 1);
@@ -478,7 +522,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   if (wg_last < 0) return;  // uniform over the workgroup
 
   // this wave's queries
-  const int unit = blockIdx.z * 4 + wave;
+  const int unit = bz * 4 + wave;
   const int half = unit / G, head = kvh * G + unit % G;
   const int q0 = half * 32;
   const bool working = unit < 2 * G && q0 < count;
@@ -516,81 +560,75 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- staging: registers <- memory, LDS <- registers
-  bf16x8_t rk[2][PER], rv[2][PER];
-  auto fetch = [&](int kb) {
+  // ---- this wave's share of the copies: piece `wave` of every step.  A piece that would start
+  // beyond the last key repeats the last one (finite numbers; its scores are masked).
+  const int kb0 = (wg_lo / 32) * 32;
+  const int nsteps = (wg_last - kb0) / 32 + 1;
+  const int last_piece = (wg_last / 16) * 16;
+  const int piece_tt = wave & 1;
+  const bool piece_is_v = wave >= 2;
+  auto page_of = [&](int step) { return table[min(kb0 + 32 * step + 16 * piece_tt, last_piece) / bs]; };
+  int page_next = page_of(0);
+  auto issue = [&](int step) {
+    const int key0 = min(kb0 + 32 * step + 16 * piece_tt, last_piece);
+    const int off0 = key0 % bs;
+    const size_t base = ((size_t)page_next * KV + kvh) * bs * D;
+    page_next = page_of(step + 1);  // a scalar load with a whole step to arrive
+    u32x4_t* dst = &lds[step % PF_STAGES][wave][0];
+    if (piece_is_v) {
+      // slot = coordinate row (slot / 2), keys 8 (slot % 2) .. + 7 of the piece
+      const bf16* src = v_pages + base + (size_t)(lane >> 1) * bs + off0 + (lane & 1) * 8;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const int key0 = kb + 16 * tt;
-      const bool live = key0 <= wg_last;
-      size_t base = 0;
-      int off0 = 0;
-      if (live) {
-        const int page = table[key0 / bs];
-        off0 = key0 % bs;
-        base = ((size_t)page * KV + kvh) * bs * D;
-      }
+      for (int i = 0; i < DC; ++i)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)i * 32 * bs), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
+    } else {
+      // slot = chunk (slot / 16) of key row (slot % 16)
+      const bf16* src = k_pages + base + (size_t)(off0 + col) * D + grp * 8;
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int c = tid + i * 256;
-        rk[tt][i] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        rv[tt][i] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        if (live && c < CHUNKS) {
-          // keys: chunk c = 8 coordinates (c % (D/8)) of key row c / (D/8)
-          rk[tt][i] = *reinterpret_cast<const bf16x8_t*>(k_pages + base + (size_t)(off0 + c / (D / 8)) * D + (c % (D / 8)) * 8);
-          // values: chunk c = 8 keys (c % 2) of coordinate row c / 2
-          rv[tt][i] = *reinterpret_cast<const bf16x8_t*>(v_pages + base + (size_t)(c / 2) * bs + off0 + (c % 2) * 8);
-        }
-      }
+      for (int i = 0; i < DC; ++i)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + i * 32), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
     }
   };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int c = tid + i * 256;
-        if (c < CHUNKS) {
-          *reinterpret_cast<bf16x8_t*>(&lds_k[buf][tt][(c / (D / 8)) * KROW + (c % (D / 8)) * 8]) = rk[tt][i];
-          *reinterpret_cast<bf16x8_t*>(&lds_v[buf][tt][(c / 2) * 16 + (c % 2) * 8]) = rv[tt][i];
-        }
-      }
-  };
-
-  int kb = (wg_lo / 32) * 32;
-  fetch(kb);
-  stash(0);
-  __syncthreads();
-  for (int buf = 0; kb <= wg_last; kb += 32, buf ^= 1) {
-    const bool more = kb + 32 <= wg_last;
-    if (more) fetch(kb + 32);
-    if (working && kb <= my_last && kb + 31 >= my_lo) {
-      // raw scores of 32 keys x 32 queries; a key operand is read from LDS once for both query tiles
-      f32x4_t sc[2][2];
+  const int nrounds = (nsteps + 1) / 2;
+  issue(0);
+  issue(1);  // beyond the last key it repeats the last piece
+  for (int rd = 0; rd < nrounds; ++rd) {
+    PF_WAIT_VM(0);    // this wave's copies for the round have landed
+    __syncthreads();  // ... and everyone's; and everyone is done with the round before
+    if (rd + 1 < nrounds) {  // into the two stages the round before used
+      issue(2 * rd + 2);
+      issue(2 * rd + 3);
+    }
+    const int kb = kb0 + 64 * rd;
+    if (working && kb <= my_last && kb + 63 >= my_lo) {
+      // raw scores of 64 keys x 32 queries; a key operand is read from LDS once for both query tiles
+      f32x4_t sc[2][4];
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) sc[qt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < 4; ++tt) sc[qt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
+      for (int tt = 0; tt < 4; ++tt) {
+        const u32x4_t* piece = &lds[(2 * rd + (tt >> 1)) % PF_STAGES][tt & 1][0];
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
-          const bf16x8_t kop = *reinterpret_cast<const bf16x8_t*>(&lds_k[buf][tt][col * KROW + c * 32 + grp * 8]);
+          const bf16x8_t kop = __builtin_bit_cast(bf16x8_t, piece[(c * 4 + grp) * 16 + col]);
 #pragma unroll
           for (int qt = 0; qt < 2; ++qt)
             sc[qt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[qt][c], sc[qt][tt], 0, 0, 0);
         }
-      // Only steps that touch the causal diagonal, the window's edge or the end of the context
-      // need a mask; the others see all 32 keys (uniform over the wave).
-      const bool masked = kb + 31 > my_first_q || (window > 0 && kb < my_last - window + 1);
-      bf16x8_t pop[2];
+      }
+      // Only rounds that touch the causal diagonal, the window's edge or the end of the context
+      // need a mask; the others see all 64 keys (uniform over the wave).
+      const bool masked = kb + 63 > my_first_q || (window > 0 && kb < my_last - window + 1);
+      bf16x8_t pop[2][2];
       float alpha[2];
       bool rescale = false;
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) {
         if (masked) {
 #pragma unroll
-          for (int tt = 0; tt < 2; ++tt)
+          for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const int key = kb + 16 * tt + 4 * grp + r;
@@ -598,32 +636,31 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
               sc[qt][tt][r] = seen ? sc[qt][tt][r] : NEG_INF;
             }
         }
-        float mx = fmaxf(fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3])),
-                         fmaxf(fmaxf(sc[qt][1][0], sc[qt][1][1]), fmaxf(sc[qt][1][2], sc[qt][1][3])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        float mx = NEG_INF;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+          mx = fmaxf(mx, fmaxf(fmaxf(sc[qt][tt][0], sc[qt][tt][1]), fmaxf(sc[qt][tt][2], sc[qt][tt][3])));
+        mx = quad_rows_max(mx);
         // base-2 softmax: scale and log2(e) are folded into one factor (positive, so maxima agree)
         const float mn = fmaxf(m[qt], mx * scale2);
         float rs = 0.f;
         alpha[qt] = 1.f;
         if (mn == NEG_INF) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pop[qt][j] = (bf16)0.f;
+          for (int j = 0; j < 8; ++j) pop[qt][0][j] = pop[qt][1][j] = (bf16)0.f;
         } else {
           alpha[qt] = __builtin_amdgcn_exp2f(m[qt] - mn);  // 2^-inf = 0 while nothing was seen
 #pragma unroll
-          for (int tt = 0; tt < 2; ++tt)
+          for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const float pv = __builtin_amdgcn_exp2f(fmaf(sc[qt][tt][r], scale2, -mn));
               rs += pv;
-              pop[qt][tt * 4 + r] = (bf16)pv;
+              pop[qt][tt >> 1][(tt & 1) * 4 + r] = (bf16)pv;
             }
           m[qt] = mn;
         }
-        rs += __shfl_xor(rs, 16, WAVE);
-        rs += __shfl_xor(rs, 32, WAVE);
-        l[qt] = l[qt] * alpha[qt] + rs;
+        l[qt] = l[qt] * alpha[qt] + quad_rows_sum(rs);
         rescale = rescale || alpha[qt] != 1.f;
       }
       // the accumulated output is rescaled only when some query's maximum moved (rare once the
@@ -635,20 +672,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
           for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha[qt];
       }
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        bf16x8_t vop;
+      for (int j = 0; j < 2; ++j) {
+        const bf16* stage_v = reinterpret_cast<const bf16*>(&lds[(2 * rd + j) % PF_STAGES][2][0]);
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-          const bf16x4_t v4 = *reinterpret_cast<const bf16x4_t*>(&lds_v[buf][tt][(dt * 16 + col) * 16 + 4 * grp]);
+        for (int dt = 0; dt < DT; ++dt) {
+          bf16x8_t vop;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
+          for (int tt = 0; tt < 2; ++tt) {
+            const bf16x4_t v4 = *reinterpret_cast<const bf16x4_t*>(stage_v + tt * (PIECE * 8) + (dt * 16 + col) * 16 + 4 * grp);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
+          }
+#pragma unroll
+          for (int qt = 0; qt < 2; ++qt) o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt][j], o[qt][dt], 0, 0, 0);
         }
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt], o[qt][dt], 0, 0, 0);
       }
     }
-    if (more) stash(buf ^ 1);
-    __syncthreads();
   }
 
 #pragma unroll
@@ -665,19 +704,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   }
 }
 
-// tiles: [num_tiles, 4] int32 (first flat token, count <= 64, block-table row, first position).
+// tiles: [num_tiles, 4] int32 (first flat token, count <= 64, block-table row, first position);
+// fastest when sorted by first position + count, largest first.
 extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, const int* tiles,
                                     int num_tiles, const int* block_tables, int table_width, void* out, int H,
                                     int KV, int D, int bs, float scale, int window, hipStream_t stream) {
   if (num_tiles <= 0) return AS_OK;
   if (H <= 0 || KV <= 0 || H % KV || bs <= 0 || table_width <= 0) return AS_BAD_SHAPE;
   const int G = H / KV;
-  if (D % 32 || D <= 0 || D > 224 || bs % 16) return AS_BAD_SHAPE;  // wider heads: tiles exceed LDS
-  dim3 grid(num_tiles, KV, (2 * G + 3) / 4);
-#define LAUNCH(DCV)                                                                                    \
-  attn_prefill_mfma_kernel<DCV><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,       \
-                                                          (const bf16*)v_pages, tiles, block_tables,  \
-                                                          table_width, (bf16*)out, H, KV, bs, scale, window)
+  if (D % 32 || D <= 0 || D > 256 || bs % 16) return AS_BAD_SHAPE;
+  const int units_z = (2 * G + 3) / 4;
+  const long items = (long)num_tiles * KV * units_z;
+  if (items > 0x7fffffffL) return AS_BAD_SHAPE;
+  const int pass = compute_units();
+#define LAUNCH(DCV)                                                                                   \
+  attn_prefill_mfma_kernel<DCV><<<(int)items, 256, 0, stream>>>(                                      \
+      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, tiles, block_tables, table_width,   \
+      (bf16*)out, H, KV, bs, scale, window, units_z, pass)
   switch (D / 32) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;
@@ -685,7 +728,8 @@ extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const vo
     case 4: LAUNCH(4); break;
     case 5: LAUNCH(5); break;
     case 6: LAUNCH(6); break;
-    default: LAUNCH(7); break;
+    case 7: LAUNCH(7); break;
+    default: LAUNCH(8); break;
   }
 #undef LAUNCH
   return launch_status();

@@ -58,3 +58,16 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 static inline int launch_status() {
   return hipGetLastError() == hipSuccess ? AS_OK : AS_LAUNCH_FAILED;
 }
+
+// Compute units of the current device (asked once per device).
+static inline int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}

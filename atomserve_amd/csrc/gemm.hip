@@ -327,18 +327,6 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
 #undef PIPE_MATH
 }
 
-static int compute_units() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 template <int NST, bool GATED>
 static int launch_pipe(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
                        hipStream_t stream) {

@@ -83,7 +83,7 @@ class StepBatch:
         bs = block_size
         tok, pos, trow, want = [], [], [], []
         slots = [[] for _ in range(num_paged_groups)]
-        short, tiles = [], []
+        short, tile_list = [], []
         row_first, row_len, row_start, row_slots = [], [], [], []
         widths = [max(1, table_width)] * num_paged_groups
         flat = 0
@@ -119,7 +119,7 @@ class StepBatch:
                 self.max_short_context = max(self.max_short_context, end)
             else:
                 for q0 in range(0, n, TILE_Q):
-                    tiles.extend((flat + q0, min(TILE_Q, n - q0), r, row.start + q0))
+                    tile_list.append((flat + q0, min(TILE_Q, n - q0), r, row.start + q0))
             self.max_context = max(self.max_context, end)
             row_first.append(flat)
             row_len.append(n)
@@ -127,6 +127,10 @@ class StepBatch:
             row_slots.append(row.state_slot)
             flat += n
 
+        # Work items of the prefill kernel, the ones that see most keys first: the kernel hands
+        # them out in this order and pairs the longest with the shortest on a compute unit.
+        tile_list.sort(key=lambda t: -(t[3] + t[1]))
+        tiles = [v for t in tile_list for v in t]
         self.max_context = max(self.max_context, max_context)
         self.max_short_context = max(self.max_short_context, max_context if short else 0)
         T, R = flat, len(rows)

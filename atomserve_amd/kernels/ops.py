@@ -189,7 +189,7 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
-PREFILL_MAX_HEAD_DIM = 224  # the staged key and value tiles of wider heads do not fit in LDS
+PREFILL_MAX_HEAD_DIM = 256  # four stages of 32 keys and values of such heads fill 128 KB of LDS
 
 
 def attn_prefill_supported(dtype, head_dim: int, block_size: int) -> bool:

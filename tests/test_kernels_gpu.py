@@ -322,7 +322,8 @@ def test_attention_serves_only_the_listed_tokens(ops):
 
 
 @pytest.mark.parametrize("H,KV,D,bs,window", [(32, 8, 128, 16, 0), (6, 2, 32, 16, 0), (8, 8, 64, 32, 0), (4, 1, 96, 16, 0),
-                                               (16, 2, 128, 16, 0), (4, 2, 64, 16, 40), (4, 2, 64, 16, 1)])  # fmt: skip
+                                               (16, 2, 128, 16, 0), (4, 2, 64, 16, 40), (4, 2, 64, 16, 1), (4, 2, 256, 16, 0),
+                                               (2, 1, 224, 32, 0), (10, 2, 160, 16, 70)])  # fmt: skip
 def test_attention_prefill(ops, H, KV, D, bs, window):
     """Prompt portions that start at position 0 and after a cached prefix, of lengths around
     the tile sizes (16, 32, 64), each query seeing keys up to its own position."""
