@@ -252,6 +252,93 @@ __global__ void qk_norm_rope_store_kernel(const O* __restrict__ qkv, const W* __
   }
 }
 
+// The same for bf16 heads that are rotated whole (R == D) and whose width is 16 times a power
+// of two: a group of D / 16 lanes owns one (token, head) and every lane moves 16-byte pieces
+// (coordinates 8l .. 8l+7 and their partners in the other half), so a wave serves several
+// heads at once and a prompt's rows move at memory speed.  Same arithmetic, same order.
+template <typename W> struct Gain8;
+template <> struct Gain8<bf16> {
+  static __device__ __forceinline__ void load(const bf16* p, float* g) {
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) g[j] = (float)v[j];
+  }
+};
+template <> struct Gain8<float> {
+  static __device__ __forceinline__ void load(const float* p, float* g) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    g[0] = a.x; g[1] = a.y; g[2] = a.z; g[3] = a.w; g[4] = b.x; g[5] = b.y; g[6] = b.z; g[7] = b.w;
+  }
+};
+
+template <typename W>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_bf16x8_kernel(
+    const bf16* __restrict__ qkv, const W* __restrict__ qw, const W* __restrict__ kw,
+    const float2* __restrict__ cs, const int* __restrict__ slots, bf16* __restrict__ q_out,
+    bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int H, int KV, int D, float eps, int block_size,
+    int heads, size_t units) {
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+  const int lpu = D >> 4, half = D >> 1;  // lanes per (token, head)
+  const size_t unit = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) / lpu;
+  const int l = threadIdx.x & (lpu - 1);
+  if (unit >= units) return;  // whole groups leave: the shuffles below stay inside a group
+  const size_t t = unit / heads;
+  const int hs = (int)(unit % heads);
+  const bf16* src = qkv + (t * (H + 2 * KV) + hs) * D;
+  const bool is_q = hs < H, is_k = !is_q && hs < H + KV;
+  const bf16x8 a8 = *reinterpret_cast<const bf16x8*>(src + 8 * l);
+  const bf16x8 b8 = *reinterpret_cast<const bf16x8*>(src + half + 8 * l);
+  bf16* dst;
+  if (is_q) {
+    dst = q_out + (t * H + hs) * D;
+  } else {
+    const int slot = slots[t];
+    if (slot < 0) return;  // uniform over the group
+    const int kvh = is_k ? hs - H : hs - H - KV;
+    const size_t head = (size_t)(slot / block_size) * KV + kvh;
+    if (!is_k) {  // values: transposed within the page
+      bf16* vt = v_pages + head * block_size * D + slot % block_size;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        vt[(size_t)(8 * l + j) * block_size] = a8[j];
+        vt[(size_t)(half + 8 * l + j) * block_size] = b8[j];
+      }
+      return;
+    }
+    dst = k_pages + (head * block_size + slot % block_size) * D;
+  }
+  const W* w = is_q ? qw : kw;
+  float inv = 1.0f;
+  if (w) {
+    float ss = 0.f;
+    // the generic kernel's order within a lane differs; the sum over D squares is the same up to rounding
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += (float)a8[j] * (float)a8[j];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += (float)b8[j] * (float)b8[j];
+    for (int off = 1; off < lpu; off <<= 1) ss += __shfl_xor(ss, off, WAVE);
+    inv = 1.0f / sqrtf(ss / (float)D + eps);
+  }
+  float ga[8], gb[8];
+  if (w) {
+    Gain8<W>::load(w + 8 * l, ga);
+    Gain8<W>::load(w + half + 8 * l, gb);
+  }
+  bf16x8 oa, ob;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float a = (float)a8[j] * inv, b = (float)b8[j] * inv;
+    if (w) { a *= ga[j]; b *= gb[j]; }
+    float c = 1.f, sn = 0.f;
+    if (cs) { const float2 v = cs[t * half + 8 * l + j]; c = v.x; sn = v.y; }
+    oa[j] = (bf16)(a * c - b * sn);
+    ob[j] = (bf16)(b * c + a * sn);
+  }
+  *reinterpret_cast<bf16x8*>(dst + 8 * l) = oa;
+  *reinterpret_cast<bf16x8*>(dst + half + 8 * l) = ob;
+}
+
 extern "C" int as_qk_norm_rope_store(const void* qkv, int dtype, const void* qw, const void* kw, int w_dtype,
                                      const float* cs, const int* slots, void* q_out, void* k_pages,
                                      void* v_pages, int num_tokens, int H, int KV, int D, int R, float eps,
@@ -259,6 +346,22 @@ extern "C" int as_qk_norm_rope_store(const void* qkv, int dtype, const void* qw,
   if (num_tokens <= 0) return AS_OK;
   if (H <= 0 || KV <= 0 || D <= 0 || R < 0 || R > D || (R & 1) || block_size <= 0) return AS_BAD_SHAPE;
   if ((qw == nullptr) != (kw == nullptr)) return AS_BAD_SHAPE;
+  const int lpu = D >> 4;
+  if (dtype == DT_BF16 && R == D && (D & 15) == 0 && lpu <= WAVE && (lpu & (lpu - 1)) == 0) {
+    const int heads = store_kv ? H + 2 * KV : H;
+    const size_t units = (size_t)num_tokens * heads;
+    const size_t blocks = (units * lpu + 255) / 256;
+    if (blocks > 0x7fffffff) return AS_BAD_SHAPE;
+#define LAUNCH8(W)                                                                                   \
+  qk_norm_rope_store_bf16x8_kernel<W><<<(int)blocks, 256, 0, stream>>>(                              \
+      (const bf16*)qkv, (const W*)qw, (const W*)kw, (const float2*)cs, slots, (bf16*)q_out,          \
+      (bf16*)k_pages, (bf16*)v_pages, H, KV, D, eps, block_size, heads, units)
+    if (w_dtype == DT_BF16) LAUNCH8(bf16);
+    else if (w_dtype == DT_F32) LAUNCH8(float);
+    else return AS_BAD_DTYPE;
+#undef LAUNCH8
+    return launch_status();
+  }
   dim3 grid(num_tokens, store_kv ? H + 2 * KV : H);
 #define LAUNCH(O, W)                                                                                   \
   qk_norm_rope_store_kernel<O, W><<<grid, WAVE, 0, stream>>>(                                          \
@@ -287,6 +390,27 @@ __global__ void silu_mul_kernel(const O* __restrict__ gu, O* __restrict__ out, i
   }
 }
 
+// The same for bf16 rows whose width is a multiple of 8: 16-byte loads and stores, which is
+// what a prompt's thousands of rows need to move at memory speed.
+__global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out,
+                                                              int inter, size_t chunks) {
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+  const int per_row = inter >> 3;
+  for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = c / per_row;
+    const int i = (int)(c % per_row) * 8;
+    const bf16x8 g8 = *reinterpret_cast<const bf16x8*>(gu + t * 2 * inter + i);
+    const bf16x8 u8 = *reinterpret_cast<const bf16x8*>(gu + t * 2 * inter + inter + i);
+    bf16x8 o8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float g = (float)g8[j];
+      o8[j] = (bf16)(g / (1.0f + expf(-g)) * (float)u8[j]);
+    }
+    *reinterpret_cast<bf16x8*>(out + t * inter + i) = o8;
+  }
+}
+
 extern "C" int as_silu_mul(const void* gate_up, void* out, int dtype, int num_tokens, int inter,
                            hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
@@ -294,6 +418,12 @@ extern "C" int as_silu_mul(const void* gate_up, void* out, int dtype, int num_to
   const size_t total = (size_t)num_tokens * inter;
   const size_t want = (total + 255) / 256;
   const int blocks = (int)(want > 8192 ? 8192 : want);
+  if (dtype == DT_BF16 && (inter & 7) == 0) {
+    const size_t chunks = total >> 3, want8 = (chunks + 255) / 256;
+    silu_mul_bf16x8_kernel<<<(int)(want8 > 16384 ? 16384 : want8), 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out,
+                                                                                    inter, chunks);
+    return launch_status();
+  }
   if (dtype == DT_F32) silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter, total);
   else if (dtype == DT_BF16) silu_mul_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, inter, total);
   else return AS_BAD_DTYPE;

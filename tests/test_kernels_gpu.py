@@ -126,6 +126,41 @@ def test_qk_norm_rope_store(ops, dtype, heads, D, bs):
     assert (k_pages.float().abs().sum(dim=(1, 3)) > 0).sum() == 5
 
 
+@pytest.mark.parametrize("D,bs,gain,rope", [(128, 16, BF16, True), (64, 32, F32, True), (256, 16, BF16, True),
+                                              (128, 16, None, True), (32, 16, F32, False)])
+def test_qk_norm_rope_store_many_tokens_bf16(ops, D, bs, gain, rope):
+    """A prompt's worth of rows through the 16-byte path: fp32 or bf16 gains, no norm, no rotation,
+    tokens whose keys are not stored, q alone."""
+    H, KV, T = 6, 2, 333
+    torch.manual_seed(13)
+    qkv = (torch.randn(T, H + 2 * KV, D, device=DEV) * 3).to(BF16)
+    qw = kw = None
+    if gain is not None:
+        qw, kw = (torch.randn(D, device=DEV) + 1).to(gain), (torch.randn(D, device=DEV) + 1).to(gain)
+    cs = None
+    if rope:
+        inv = (1.0 / (1e6 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))).to(DEV)
+        cs = torch.empty(T, D // 2, 2, device=DEV)
+        ops.rope_table(i32(list(range(1000, 1000 + T))), inv, cs)
+    pages = -(-T // bs) + 1
+    perm = torch.randperm(pages * bs)[:T].tolist()
+    perm[7] = perm[100] = -1
+    slots = i32(perm)
+    k_pages = torch.zeros(pages, KV, bs, D, dtype=BF16, device=DEV)
+    v_pages = torch.zeros(pages, KV, D, bs, dtype=BF16, device=DEV)
+    q = torch.empty(T, H, D, dtype=BF16, device=DEV)
+    ops.qk_norm_rope_store(qkv, qw, kw, cs, slots, q, k_pages, v_pages, H, KV, 1e-6)
+    rq, rk, rv = pk.qk_norm_rope(qkv, qw, kw, cs, H, KV, 1e-6)
+    ref_k, ref_v = torch.zeros(pages, KV, bs, D, device=DEV), torch.zeros(pages, KV, D, bs, device=DEV)
+    keep = [i for i, sl in enumerate(perm) if sl >= 0]
+    pk.store_pages(ref_k, ref_v, rk[keep], rv[keep], i32([perm[i] for i in keep]))
+    assert close_bf16(q, rq) and close_bf16(k_pages, ref_k)
+    assert torch.equal(v_pages.float(), ref_v)
+    q2 = torch.empty_like(q)
+    ops.qk_norm_rope_store(qkv, qw, kw, cs, None, q2, None, None, H, KV, 1e-6, store_kv=False)
+    assert torch.equal(q2, q)
+
+
 def test_qk_norm_rope_store_variants(ops):
     """No norm, no rotation, a rotation of part of the head, and q alone (a run that reads
     another run's cache stores nothing)."""
@@ -150,7 +185,7 @@ def test_qk_norm_rope_store_variants(ops):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("rows,inter", [(1, 3072), (7, 3072), (300, 3072), (5, 160)])
+@pytest.mark.parametrize("rows,inter", [(1, 3072), (7, 3072), (300, 3072), (5, 160), (33, 100), (2048, 1536)])
 def test_silu_mul(ops, dtype, rows, inter):
     # sizes from reference tests/test_kernels.py:192-198
     torch.manual_seed(5)
