@@ -144,7 +144,9 @@ class CacheManager:
         """Give back everything the request holds (finish, abort or preemption)."""
         for g, table in zip(self.paged_groups, rc.tables):
             g.allocator.free([p for p in table if p != RELEASED])
-            table.clear()
+        # new lists, not cleared ones: whoever still holds the old tables (a step packed earlier)
+        # can tell that they no longer describe this request
+        rc.tables = [[] for _ in self.paged_groups]
         rc.hashes.clear()
         if rc.state_slot >= 0:
             self._free_slots.append(rc.state_slot)

@@ -337,6 +337,112 @@ extern "C" int as_sample(const float* logits, int B, int V, const float* tempera
   return launch_status();
 }
 
+// ---- the same draw for small top-k, spread over the GPU ---------------------------------
+// One workgroup per row reads a vocabulary of 150 thousand logits alone, which takes longer
+// than everything else a decode step does after its last matrix product.  When every row
+// keeps at most SPLIT_KMAX candidates, the row is cut into SPLIT_SLICES slices instead:
+// a first kernel finds each slice's k best (keys carry the index within the whole row), a
+// second one ranks the slices' candidates, of which the row's k best are a subset, and
+// draws exactly as sample_kernel does: same candidates, same order, same noise.
+#define SPLIT_SLICES 32
+#define SPLIT_KMAX 64
+#define SPLIT_THREADS 256
+
+__device__ __forceinline__ int effective_top_k(float T, int k, float p_keep) {
+  return (T <= 0.f || p_keep <= 0.f) ? 1 : k;  // greedy: the best token alone
+}
+
+__global__ __launch_bounds__(SPLIT_THREADS) void topk_slices_kernel(
+    const float* __restrict__ logits, int V, const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, unsigned long long* __restrict__ cand, int* __restrict__ counts) {
+  __shared__ TopKShared topk_shared;
+  __shared__ unsigned long long sel[SPLIT_KMAX];
+  const int row = blockIdx.x, slice = blockIdx.y;
+  int k = effective_top_k(temperature[row], top_k[row], top_p[row]);
+  k = k < 1 ? 1 : (k > SPLIT_KMAX ? SPLIT_KMAX : k);  // refused on the host; never index outside
+  const int len = (V + SPLIT_SLICES - 1) / SPLIT_SLICES, off = slice * len;
+  const int n = min(len, V - off);
+  int found = 0;
+  if (n > 0) found = block_topk(logits + (size_t)row * V + off, n, min(k, n), sel, topk_shared);
+  unsigned long long* dst = cand + ((size_t)row * SPLIT_SLICES + slice) * SPLIT_KMAX;
+  for (int r = threadIdx.x; r < found; r += SPLIT_THREADS) dst[r] = make_key(key_value(sel[r]), key_index(sel[r]) + off);
+  if (threadIdx.x == 0) counts[row * SPLIT_SLICES + slice] = found;
+}
+
+__global__ __launch_bounds__(SPLIT_THREADS) void sample_candidates_kernel(
+    const unsigned long long* __restrict__ cand, const int* __restrict__ counts,
+    const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const long long* __restrict__ seeds, const int* __restrict__ counters, int* __restrict__ out) {
+  __shared__ unsigned long long pool[SPLIT_SLICES * SPLIT_KMAX];
+  __shared__ int first[SPLIT_SLICES + 1];
+  __shared__ unsigned long long sel[SPLIT_KMAX];
+  __shared__ float ework[SPLIT_KMAX];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  float T = temperature[row];
+  const float p_keep = top_p[row];
+  int k = effective_top_k(T, top_k[row], p_keep);
+  if (T <= 0.f || p_keep <= 0.f) T = 1.f;
+  k = k < 1 ? 1 : (k > SPLIT_KMAX ? SPLIT_KMAX : k);
+  if (tid == 0) {
+    int at = 0;
+    for (int sl = 0; sl < SPLIT_SLICES; ++sl) { first[sl] = at; at += counts[row * SPLIT_SLICES + sl]; }
+    first[SPLIT_SLICES] = at;
+  }
+  __syncthreads();
+  const int total = first[SPLIT_SLICES];
+  for (int sl = tid / SPLIT_KMAX; sl < SPLIT_SLICES; sl += SPLIT_THREADS / SPLIT_KMAX) {
+    const int r = tid % SPLIT_KMAX, n = first[sl + 1] - first[sl];
+    if (r < n) pool[first[sl] + r] = cand[((size_t)row * SPLIT_SLICES + sl) * SPLIT_KMAX + r];
+  }
+  __syncthreads();
+  for (int c = tid; c < total; c += SPLIT_THREADS) {
+    const unsigned long long key = pool[c];
+    int rank = 0;
+    for (int j = 0; j < total; ++j) rank += pool[j] > key;
+    if (rank < k) sel[rank] = key;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    const int found = total < k ? total : k;
+    const long long seed = seeds[row];
+    const int counter = counters[row];
+    int choice = 0;
+    if (found > 1) {
+      const float v0 = key_value(sel[0]);
+      float sum = 0.f;
+      for (int i = 0; i < found; ++i) {
+        const float e = expf((key_value(sel[i]) - v0) / T);
+        ework[i] = e;
+        sum += e;
+      }
+      float mass = 0.f, best_score = -1.f;
+      for (int i = 0; i < found; ++i) {
+        const float p = ework[i] / sum;
+        if (mass >= p_keep) break;  // the mass ranked above already reaches top_p
+        mass += p;
+        const float score = p / exp1_noise(seed, counter, i);
+        if (score > best_score) { best_score = score; choice = i; }
+      }
+    }
+    out[row] = found ? key_index(sel[choice]) : 0;
+  }
+}
+
+// As as_sample, for batches whose every row keeps between 1 and 64 candidates (greedy rows
+// count as 1).  cand: [B, 32, 64] 64-bit scratch, counts: [B, 32] int32 scratch.
+extern "C" int as_sample_split(const float* logits, int B, int V, const float* temperature, const int* top_k,
+                               const float* top_p, const long long* seeds, const int* counters, void* cand,
+                               int* counts, int* out, hipStream_t stream) {
+  if (B <= 0) return AS_OK;
+  if (V <= 0 || !cand || !counts) return AS_BAD_SHAPE;
+  topk_slices_kernel<<<dim3(B, SPLIT_SLICES), SPLIT_THREADS, 0, stream>>>(logits, V, temperature, top_k, top_p,
+                                                                         (unsigned long long*)cand, counts);
+  if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
+  sample_candidates_kernel<<<B, SPLIT_THREADS, 0, stream>>>((const unsigned long long*)cand, counts, temperature,
+                                                            top_k, top_p, seeds, counters, out);
+  return launch_status();
+}
+
 // Sorted top-k of each row (values and indices), k <= SAMPLE_KMAX; exposed for tests and tools.
 __global__ __launch_bounds__(SAMPLE_THREADS) void topk_kernel(const float* __restrict__ logits, int V, int k,
                                                               float* __restrict__ values, int* __restrict__ indices) {

@@ -170,10 +170,13 @@ class StepBatch:
             staging.sent()
         self._host = host  # alive until the copy has run
         self.device_buffer, self.layout = dev, sizes
-        offset, parts = 0, {}
+        offset, parts, self._at = 0, {}, {}
         for (name, _), a in zip(fields, arrays):
             parts[name] = dev[offset : offset + a.size]
+            self._at[name] = offset
             offset += a.size
+        self._packed = np.concatenate(arrays) if total else np.zeros(0, dtype=np.int32)  # what `advance` edits
+        self._staging, self._widths, self._vocab = staging, widths, vocab_size
 
         self.num_tokens, self.num_rows = T, R
         self.token_ids, self.positions, self.tok_row = parts["token_ids"], parts["positions"], parts["tok_row"]
@@ -189,6 +192,47 @@ class StepBatch:
         self.block_size = bs
         self.pools = pools
         self.shared = {}  # per-step results that parts share (rotary tables, ...)
+
+    def advance(self, rows) -> bool:
+        """The next decode step of the same requests, in place: every row brings the one token
+        that follows the row packed last, from the same block tables, so only the token, its
+        position, its slots and the table entry of its page change.  Uploads and returns True,
+        or returns False and changes nothing if `rows` are anything else (pack them anew)."""
+        old_rows, bs = self.host_rows, self.block_size
+        if len(rows) != len(old_rows) or self.num_tokens != len(old_rows):
+            return False
+        for new, old in zip(rows, old_rows):
+            if (len(new.tokens) != 1 or new.tables is not old.tables or new.store != old.store or new.want != old.want
+                    or new.state_slot != old.state_slot or new.start != old.start + (1 if new.store else 0)):
+                return False
+            if not 0 <= new.tokens[0] < self._vocab:
+                return False  # the full packing names the error
+            for g, table in enumerate(new.tables):
+                page = new.start // bs
+                if page >= self._widths[g] or page >= len(table) or table[page] == RELEASED:
+                    return False
+        p, at = self._packed, self._at
+        for r, row in enumerate(rows):
+            p[at["token_ids"] + r] = row.tokens[0]
+            p[at["positions"] + r] = row.start
+            p[at["row_start"] + r] = row.start
+            for g, table in enumerate(row.tables):
+                page = row.start // bs
+                p[at[f"slots{g}"] + r] = table[page] * bs + row.start % bs if row.store else -1
+                p[at[f"tables{g}"] + r * self._widths[g] + page] = table[page]
+        total = p.size
+        if self._staging is not None:
+            host = self._staging.take(total)
+        else:
+            host = torch.empty(total, dtype=torch.int32, pin_memory=self.device_buffer.is_cuda)
+        host.numpy()[:total] = p
+        self.device_buffer.copy_(host[:total], non_blocking=True)
+        if self._staging is not None:
+            self._staging.sent()
+        self._host = host
+        self.host_rows = rows
+        self.shared = {}
+        return True
 
     def cache_view(self, cache_id: int, writes: bool):
         """The view of cache `cache_id` for a mixer in this step."""

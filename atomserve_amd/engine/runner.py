@@ -53,6 +53,7 @@ class DecodeGraphs:
     def __init__(self, runner):
         self.runner = runner
         self.graphs = {}
+        self.filler_tables = [[0] for _ in runner.manager.paged_groups]  # one object: a filler row is recognised
 
     def eligible(self, rows) -> bool:
         r = self.runner
@@ -70,9 +71,8 @@ class DecodeGraphs:
         longest = max(row.start + 1 for row in rows)
         context = -(-longest // self.CONTEXT_STEP) * self.CONTEXT_STEP
         width = -(-context // bs)
-        filler = Row([0], 0, [[0] for _ in r.manager.paged_groups], [], -1, store=False)
         padded = [Row(row.tokens, row.start, row.tables, [0], row.state_slot) for row in rows] + [
-            Row(filler.tokens, 0, filler.tables, [0], -1, store=False) for _ in range(n - len(rows))
+            Row([0], 0, self.filler_tables, [0], -1, store=False) for _ in range(n - len(rows))
         ]
         key = (n, context)
         entry = self.graphs.get(key)
@@ -99,8 +99,10 @@ class DecodeGraphs:
                 if collecting:
                     gc.enable()
             entry = self.graphs[key] = (graph, batch, logits)
-        else:
-            r.prepare(padded, table_width=width, max_context=context, into=entry[1])
+        elif not entry[1].advance(padded):
+            # other requests than last time, or a window moved: pack anew into the captured buffer
+            batch = r.prepare(padded, table_width=width, max_context=context, into=entry[1])
+            entry = self.graphs[key] = (entry[0], batch, entry[2])
         graph, batch, logits = entry
         graph.replay()
         wanted = [i for i, row in enumerate(rows) if row.want]

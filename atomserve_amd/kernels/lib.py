@@ -31,6 +31,7 @@ SIGNATURES = {
     "as_gemm_bf16_gated": ("gemm", [P, P, P, I, I, I, I, P]),
     "as_argmax": ("sampling", [P, P, I, I, P]),
     "as_sample": ("sampling", [P, I, I, P, P, P, P, P, P, P]),
+    "as_sample_split": ("sampling", [P, I, I, P, P, P, P, P, P, P, P, P]),
     "as_apply_penalty": ("sampling", [P, P, P, P, I, I, P]),
     "as_topk": ("sampling", [P, I, I, I, P, P, P]),
 }

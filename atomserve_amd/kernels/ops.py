@@ -290,12 +290,17 @@ def apply_penalty(logits, rows, cols, amounts) -> None:
     call("as_apply_penalty", _ptr(logits), _ptr(rows), _ptr(cols), _ptr(amounts), n, logits.shape[1], _stream())
 
 
-def sample(logits, temperature, top_k, top_p, seeds, counters, out) -> None:
+SAMPLE_SPLIT_MAX_TOP_K = 64  # up to here a row's candidates are found by 32 workgroups instead of one
+
+
+def sample(logits, temperature, top_k, top_p, seeds, counters, out, max_top_k=None) -> None:
     """One token per row: top-k (0: all), temperature (0: greedy), top-p, seeded draw.
 
     temperature, top_p fp32 [B]; top_k, counters int32 [B]; seeds int64 [B]; out int32 [B].
     top_k values must be 0 (or >= vocabulary) or at most SAMPLE_MAX_TOP_K; checked by the caller
-    on the host values it uploads."""
+    on the host values it uploads.  max_top_k: the caller's promise that every row keeps between 1
+    and this many candidates (a greedy row keeps 1); up to SAMPLE_SPLIT_MAX_TOP_K the rows are
+    then searched by many workgroups each, with the same result."""
     _check(logits, "logits", F32, (None, None))
     B = logits.shape[0]
     _check(temperature, "temperature", F32, (B,))
@@ -304,6 +309,12 @@ def sample(logits, temperature, top_k, top_p, seeds, counters, out) -> None:
     _check(seeds, "seeds", torch.int64, (B,))
     _check(counters, "counters", I32, (B,))
     _check(out, "out", I32, (B,))
+    if max_top_k is not None and 1 <= max_top_k <= SAMPLE_SPLIT_MAX_TOP_K:
+        cand = torch.empty((B, 32, SAMPLE_SPLIT_MAX_TOP_K), dtype=torch.int64, device=logits.device)
+        counts = torch.empty((B, 32), dtype=I32, device=logits.device)
+        call("as_sample_split", _ptr(logits), B, logits.shape[1], _ptr(temperature), _ptr(top_k), _ptr(top_p),
+             _ptr(seeds), _ptr(counters), _ptr(cand), _ptr(counts), _ptr(out), _stream())  # fmt: skip
+        return
     call("as_sample", _ptr(logits), B, logits.shape[1], _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
          _ptr(counters), _ptr(out), _stream())  # fmt: skip
 

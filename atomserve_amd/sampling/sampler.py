@@ -10,6 +10,7 @@ candidate), so a request's stream does not depend on its batch neighbours; reque
 without a seed get one drawn by the engine when they are submitted.
 """
 
+import numpy as np
 import torch
 
 from atomserve_amd.kernels import ops
@@ -37,17 +38,26 @@ class Sampler:
         if all(p.temperature == 0 for p in params):
             ops.argmax(logits, out)
             return out.tolist()
-        top_k = []
+        top_k, kept = [], []
         for p in params:
             k = p.top_k if 0 < p.top_k < vocab else 0
             if k > ops.SAMPLE_MAX_TOP_K:
                 raise ValueError(f"top_k {k} is beyond the kernel's {ops.SAMPLE_MAX_TOP_K}; use 0 for all tokens")
             top_k.append(k)
-        floats = torch.tensor([[max(p.temperature, 0.0) for p in params], [p.top_p for p in params]],
-                              dtype=torch.float32).to(self.device, non_blocking=True)  # fmt: skip
-        ints = torch.tensor([top_k, [len(s.output_ids) for s in seqs]], dtype=torch.int32).to(self.device, non_blocking=True)
-        seeds = torch.tensor([_as_int64(s.noise_seed) for s in seqs], dtype=torch.int64).to(self.device, non_blocking=True)
-        ops.sample(logits, floats[0], ints[0], floats[1], seeds, ints[1], out)
+            # candidates the row keeps; all tokens (k == 0) is left to the one-workgroup kernel
+            kept.append(1 if p.temperature <= 0 or p.top_p <= 0 else (k or ops.SAMPLE_MAX_TOP_K + 1))
+        # One upload: int32 rows (temperature and top_p as their bit patterns, top_k, tokens sampled
+        # so far), then the 64-bit seeds.
+        host = np.empty(6 * B, dtype=np.int32)
+        host[0:B].view(np.float32)[:] = [max(p.temperature, 0.0) for p in params]
+        host[B : 2 * B].view(np.float32)[:] = [p.top_p for p in params]
+        host[2 * B : 3 * B] = top_k
+        host[3 * B : 4 * B] = [len(s.output_ids) for s in seqs]
+        host[4 * B :].view(np.int64)[:] = [_as_int64(s.noise_seed) for s in seqs]
+        dev = torch.from_numpy(host).to(self.device, non_blocking=True)
+        floats, ints = dev[: 2 * B].view(torch.float32), dev[2 * B : 4 * B]
+        ops.sample(logits, floats[:B], ints[:B], floats[B:], dev[4 * B :].view(torch.int64), ints[B:], out,
+                   max_top_k=max(kept))  # fmt: skip
         return out.tolist()
 
     def _apply_presence_penalty(self, logits, seqs):

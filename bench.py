@@ -117,13 +117,17 @@ def main() -> int:
     result_prefill = None
     if not args.no_prefill:
         one = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
-        engine.generate([prompt(99, 2048, c.vocab_size)], one)  # warm-up
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        engine.generate([prompt(98, 2048, c.vocab_size)], one)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
         T = 2048
+        for i in range(2):  # warm-up: libraries pick their kernels, pools are touched
+            engine.generate([prompt(99 - i, T, c.vocab_size)], one)
+        times = []
+        for i in range(3):  # different prompts, nothing reused; the median of three
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.generate([prompt(90 + i, T, c.vocab_size)], one)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        dt = sorted(times)[1]
         flops = 2 * T * layer_params * c.num_layers + 2 * c.hidden_size * c.vocab_size \
             + 4 * c.num_heads * c.head_dim * (T * (T + 1) // 2) * c.num_layers  # fmt: skip
         result_prefill = {"value": round(T / dt, 1), "tokens": T, "ms": round(dt * 1e3, 3),

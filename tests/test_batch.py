@@ -1,0 +1,68 @@
+"""The flat batch of a step on the host side: what is packed, and the in-place update of a
+repeated decode step."""
+
+import pytest
+import torch
+
+from atomserve_amd.cache.manager import RELEASED
+from atomserve_amd.engine.batch import Row, StepBatch
+
+BS = 4
+
+
+def pack(rows, **layout):
+    return StepBatch(rows, BS, 2, 100, "cpu", **layout)
+
+
+def decode_rows(tables, starts, tokens, filler):
+    rows = [Row([t], s, tb, [0], -1) for tb, s, t in zip(tables, starts, tokens)]
+    return rows + [Row([0], 0, filler, [0], -1, store=False)]
+
+
+def test_rows_are_flattened_with_slots_tables_and_tiles():
+    t0, t1 = [[5, 2], [7, 1]], [[3], [4]]
+    b = pack([Row([11, 12, 13], 4, t0, [2]), Row([21], 2, t1, [0])])
+    assert b.token_ids.tolist() == [11, 12, 13, 21] and b.positions.tolist() == [4, 5, 6, 2]
+    assert b.tok_row.tolist() == [0, 0, 0, 1] and b.logits_rows.tolist() == [2, 3]
+    assert b.group_slots[0].tolist() == [2 * BS + 0, 2 * BS + 1, 2 * BS + 2, 3 * BS + 2]
+    assert b.group_slots[1].tolist() == [1 * BS + 0, 1 * BS + 1, 1 * BS + 2, 4 * BS + 2]
+    assert b.group_tables[0].tolist() == [[5, 2], [3, 0]]
+    assert b.short_tokens.tolist() == [0, 1, 2, 3] and b.num_long_tiles == 0
+    long = pack([Row(list(range(70)), 0, [list(range(20)), list(range(20))], []), Row([1] * 9, 64, [list(range(20, 40))] * 2, [])])
+    # work items of the prefill kernel, the one that sees most keys first
+    assert long.long_tiles.tolist() == [[70, 9, 1, 64], [64, 6, 0, 64], [0, 64, 0, 0]]
+
+
+def test_a_repeated_decode_step_is_updated_in_place():
+    """Same requests, one position further: `advance` leaves exactly what packing anew gives, also
+    when a request has just received a new page; anything else is refused untouched."""
+    filler = [[0], [0]]
+    tables = [[[5, 2], [7, 1]], [[3], [4]]]  # request 0 at position 6, request 1 at position 3 (last slot of its page)
+    layout = dict(table_width=3, max_context=12)
+    first = pack(decode_rows(tables, [6, 3], [11, 21], filler), **layout)
+    batch = pack(decode_rows(tables, [6, 3], [11, 21], filler), into=first, **layout)
+    tables[1][0].append(8)  # request 1 crosses into a new page
+    tables[1][1].append(9)
+    rows = decode_rows(tables, [7, 4], [12, 22], filler)
+    assert batch.advance(rows)
+    fresh = pack(decode_rows(tables, [7, 4], [12, 22], filler), **layout)
+    assert torch.equal(first.device_buffer, fresh.device_buffer)  # `first` owns the buffer both wrote to
+    assert batch.host_rows is rows and batch.shared == {}
+    before = first.device_buffer.clone()
+    for bad in (
+        decode_rows(tables, [9, 5], [1, 2], filler),                      # a position was skipped
+        decode_rows([tables[1], tables[0]], [8, 5], [1, 2], filler),      # other requests in these rows
+        decode_rows([[list(t) for t in tables[0]], tables[1]], [8, 5], [1, 2], filler),  # equal tables, another object
+        decode_rows(tables, [8, 5], [1, 2], [[0], [0]]),                  # not the filler it was packed with
+        decode_rows(tables, [8, 5], [1, 2], filler)[:2],                  # fewer rows
+        [Row([1, 2], 8, tables[0], [0], -1), *decode_rows(tables, [8, 5], [1, 2], filler)[1:]],  # two tokens
+        decode_rows(tables, [8, 5], [1, 200], filler),                    # a token outside the vocabulary
+    ):
+        assert not batch.advance(bad)
+        assert torch.equal(first.device_buffer, before)
+    tables[0][0].append(RELEASED)
+    tables[0][1].append(6)
+    assert not batch.advance(decode_rows(tables, [8, 5], [1, 2], filler))  # its page is not there
+    tables[0][0][2] = 6
+    assert batch.advance(decode_rows(tables, [8, 5], [1, 2], filler))
+    assert not batch.advance(decode_rows(tables, [12, 6], [1, 2], filler))  # beyond the packed table width

@@ -447,13 +447,13 @@ def test_topk_matches_the_library(ops):
             assert torch.equal(x.gather(1, indices.long().clamp_min(0)), expected)
 
 
-def sample_rows(ops, logits, temperature, top_k, top_p, seeds, counters=None):
+def sample_rows(ops, logits, temperature, top_k, top_p, seeds, counters=None, max_top_k=None):
     B = logits.shape[0]
     out = torch.empty(B, dtype=I32, device=DEV)
     f = lambda v: torch.full((B,), v, dtype=F32, device=DEV) if not torch.is_tensor(v) else v  # noqa: E731
     ops.sample(logits, f(temperature), torch.full((B,), top_k, dtype=I32, device=DEV) if not torch.is_tensor(top_k) else top_k,
                f(top_p), torch.as_tensor(seeds, dtype=torch.int64).to(DEV),
-               torch.zeros(B, dtype=I32, device=DEV) if counters is None else counters, out)  # fmt: skip
+               torch.zeros(B, dtype=I32, device=DEV) if counters is None else counters, out, max_top_k=max_top_k)  # fmt: skip
     return out
 
 
@@ -478,6 +478,27 @@ def test_sampling_follows_the_distribution(ops):
         assert set(sample_rows(ops, logits[:200], 1.0, top_k, 0.01, seeds[:200]).tolist()) == {0}
     sharp = sample_rows(ops, logits, 0.5, 0, 1.0, seeds).long().bincount(minlength=4).float().cpu() / n
     assert torch.allclose(sharp, PROBS**2 / (PROBS**2).sum(), atol=0.015)
+
+
+@pytest.mark.parametrize("V", [151936, 4097, 100, 31])
+def test_sampling_split_over_workgroups_draws_the_same_tokens(ops, V):
+    """Rows that keep few candidates are searched by many workgroups: the same tokens as the
+    one-workgroup kernel, also among equal logits (the lower index ranks first), with greedy
+    rows, every top-p and fewer tokens than slices."""
+    torch.manual_seed(14)
+    B = 24
+    logits = torch.randn(B, V, device=DEV) * 3
+    logits[B // 2 :] = (logits[B // 2 :] * 2).round() / 2  # long runs of equal values
+    logits[3, V // 3] = float("nan")
+    top_k = i32([(1, 2, 20, 33, 64)[i % 5] if (1, 2, 20, 33, 64)[i % 5] < V else V - 1 for i in range(B)])
+    temperature = torch.tensor([(1.0, 0.6, 0.0, 1.5)[i % 4] for i in range(B)], device=DEV)
+    top_p = torch.tensor([(1.0, 0.95, 0.5, 0.0, 0.01)[i % 5] for i in range(B)], device=DEV)
+    seeds = torch.arange(B) * 104729 + 5
+    for c in range(4):
+        counters = i32([c] * B)
+        one = sample_rows(ops, logits, temperature, top_k, top_p, seeds, counters)
+        many = sample_rows(ops, logits, temperature, top_k, top_p, seeds, counters, max_top_k=64)
+        assert torch.equal(one, many)
 
 
 def test_sampling_is_seeded_per_request_and_mixes_greedy_rows(ops):
