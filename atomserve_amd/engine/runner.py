@@ -44,10 +44,11 @@ class DecodeGraphs:
     A decode step is some hundred small launches; issuing them from the host costs more than
     running them.  For each (rows rounded up, context rounded up) one pass is captured; later
     steps copy their integers into the captured step's buffer and replay it.  Rows that pad a
-    step to its bucket store nothing and their logits are dropped.  Only kernels of this
-    package are captured (up to GRAPH_MAX_ROWS rows the matrix products are our own too)."""
+    step to its bucket store nothing and their logits are dropped.  Up to 16 rows every captured
+    kernel is this package's; above, the matrix products are the library's, which replay
+    correctly (checked against eager steps in the tests, several replays with eager work between)."""
 
-    ROW_BUCKETS = (1, 2, 4, 8, 16)
+    ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64)
     CONTEXT_STEP = 1024
 
     def __init__(self, runner):

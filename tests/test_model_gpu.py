@@ -82,6 +82,55 @@ def test_first_tokens_and_long_decoding(setup, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("num_requests", [3, 13, 40])
+def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
+    """Decode steps replayed as captured graphs against the same steps launched kernel by kernel:
+    the same logits at every step, over several replays with eager work (a new request's prompt)
+    and synchronisations between them, for row counts in the small buckets and the large ones
+    (whose matrix products are the library's)."""
+    from atomserve_amd.cache.manager import CacheManager
+    from atomserve_amd.engine.batch import Row
+    from atomserve_amd.engine.runner import ModelRunner
+    from atomserve_amd.weights.loader import load_model
+
+    name, raw, weights, path, cache = setup
+    model, _, _ = load_model(path, getattr(torch, dtype), "cuda:0")
+    vocab = raw["vocab_size"]
+    prompts = [rc.random_ids(vocab, 5 + 3 * (i % 11), seed=300 + i) for i in range(num_requests)]
+    later = [rc.random_ids(vocab, 12, seed=400 + i) for i in range(num_requests)]  # the tokens decoded, given
+    extra = rc.random_ids(vocab, 40, seed=500)
+    seen = {}
+    for use_graphs in (True, False):
+        manager = CacheManager(model.cache_requests(), 16, 8 * num_requests + 16, num_requests + 2)
+        runner = ModelRunner(model, manager, use_graphs=use_graphs)
+        live = [[manager.new_request(), 0] for _ in range(num_requests)]
+
+        def rows_of(token_lists, who=live):
+            rows = []
+            for state, tokens in zip(who, token_lists):
+                assert manager.reserve(state[0], state[1], len(tokens))
+                rows.append(Row(list(tokens), state[1], state[0].tables, [len(tokens) - 1], state[0].state_slot))
+                state[1] += len(tokens)
+            return rows
+
+        out = [runner.step(rows_of(prompts)).float().cpu()]
+        for step in range(8):
+            if step == 3:  # eager work between the replays: another request's prompt, alone in its step
+                other = [[manager.new_request(), 0]]
+                out.append(runner.step(rows_of([extra], other)).float().cpu())
+                torch.cuda.synchronize()
+            out.append(runner.step(rows_of([[t[step]] for t in later])).float().cpu())
+        if use_graphs and dtype in ("float32", "bfloat16"):
+            assert runner.decode_graphs.graphs, "no step was replayed from a graph"
+        seen[use_graphs] = out
+    # a replayed step is padded to its bucket and cuts contexts by the bucket's bound, so sums are
+    # taken in another order: the same numbers up to rounding
+    for a, b in zip(seen[True], seen[False]):
+        assert a.shape == b.shape and torch.isfinite(a).all()
+        check(float((a - b).abs().max()), float(b.abs().max()), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(setup, dtype, tmp_path):
     """The program itself, as a user starts it: JSON lines in, <step>.f32 files and `done` lines out."""
     name, raw, weights, path, cache = setup
