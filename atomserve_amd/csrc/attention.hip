@@ -444,15 +444,16 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 // of 32 keys.  A round of the main loop computes 64 keys (two stages) while the copies of the
 // next 64 are in flight into the other two, and costs one barrier; 64 keys give a wave 64
 // independent MFMAs between its softmax reductions, which is what hides their latency.
-// Each wave copies one of a stage's four 16-key pieces (keys 0-15, keys 16-31, values 0-15,
-// values 16-31): such a piece of a page is contiguous in memory both for keys and, thanks
-// to the transposed value pages, for values.
+// Two waves copy a stage's keys, two its values (a 16-key piece of a page is contiguous in
+// memory both for keys and, thanks to the transposed value pages, for values).
 //
-// LDS layout of a piece, in 16-byte slots:
-//   keys:   slot (c * 16 + r) holds coordinates 8c .. 8c+7 of key row r, so the 64 lanes of
-//           an MFMA operand read (row = lane % 16, chunk = 4 step + lane / 16) touch 64
-//           consecutive slots: no bank conflicts, no padding, any head width;
-//   values: the page's own order [coordinate][16 keys].
+// LDS layout of a stage, in 16-byte slots:
+//   keys:   slot (chunk * 32 + t) holds coordinates 8 chunk .. + 7 of the key behind row t % 16
+//           of score tile t / 16, so the 64 lanes of an MFMA operand (row = lane % 16,
+//           chunk = 4 step + lane / 16) read four runs of 16 consecutive slots: no bank
+//           conflicts, no padding, any head width;
+//   values: per 16-key piece, slot (h * D + d) holds keys 8h .. 8h+7 of coordinate d: the eight
+//           keys whose weights a lane holds are one slot, and 16 lanes read 256 consecutive bytes.
 // A load instruction fills 64 consecutive slots (slot = first + lane); which 16 bytes of
 // memory a lane fetches is free, which is how the key layout comes about.
 // A query at position p sees keys lo..p by absolute position, wherever the row starts.
@@ -474,6 +475,10 @@ __device__ __forceinline__ float quad_rows_sum(float v) {
 }
 
 #define PF_STAGES 4
+// Which of a step's 32 keys row `row` of its score tile `tile` (0, 1) stands for.  Rows 4g..4g+3
+// of both tiles are what lane group g holds after the score product, and they are keys
+// 8g .. 8g+7: eight neighbours, whose values are one 16-byte piece of a transposed page.
+#define PF_KEY_OF_ROW(tile, row) (8 * ((row) >> 2) + ((row) & 3) + 4 * (tile))
 // s_waitcnt that only constrains the vector-memory counter (vmcnt: bits 3:0 and 15:14)
 #define PF_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
 
@@ -560,33 +565,44 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- this wave's share of the copies: piece `wave` of every step.  A piece that would start
-  // beyond the last key repeats the last one (finite numbers; its scores are masked).
+  // ---- this wave's share of the copies: of every 32-key step, waves 0 and 1 bring the keys
+  // (half of the 16-byte chunks of all 32 rows each), waves 2 and 3 the values of keys 0-15 and
+  // 16-31.  A 16-key piece that would start beyond the last key repeats the last one (finite
+  // numbers; its scores are masked).
   const int kb0 = (wg_lo / 32) * 32;
   const int nsteps = (wg_last - kb0) / 32 + 1;
   const int last_piece = (wg_last / 16) * 16;
-  const int piece_tt = wave & 1;
-  const bool piece_is_v = wave >= 2;
-  auto page_of = [&](int step) { return table[min(kb0 + 32 * step + 16 * piece_tt, last_piece) / bs]; };
-  int page_next = page_of(0);
+  auto page_of = [&](int step, int piece) { return table[min(kb0 + 32 * step + 16 * piece, last_piece) / bs]; };
+  int page_next[2] = {page_of(0, 0), page_of(0, 1)};
   auto issue = [&](int step) {
-    const int key0 = min(kb0 + 32 * step + 16 * piece_tt, last_piece);
-    const int off0 = key0 % bs;
-    const size_t base = ((size_t)page_next * KV + kvh) * bs * D;
-    page_next = page_of(step + 1);  // a scalar load with a whole step to arrive
-    u32x4_t* dst = &lds[step % PF_STAGES][wave][0];
-    if (piece_is_v) {
-      // slot = coordinate row (slot / 2), keys 8 (slot % 2) .. + 7 of the piece
-      const bf16* src = v_pages + base + (size_t)(lane >> 1) * bs + off0 + (lane & 1) * 8;
+    size_t base[2];
+    int off0[2];
 #pragma unroll
-      for (int i = 0; i < DC; ++i)
-        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + (size_t)i * 32 * bs), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
+    for (int pc = 0; pc < 2; ++pc) {
+      off0[pc] = min(kb0 + 32 * step + 16 * pc, last_piece) % bs;
+      base[pc] = ((size_t)page_next[pc] * KV + kvh) * bs * D;
+      page_next[pc] = page_of(step + 1, pc);  // scalar loads with a whole step to arrive
+    }
+    if (wave >= 2) {
+      // values of one piece: slot = h * D + d holds keys 8h .. 8h+7 of coordinate d
+      const int pc = wave - 2;
+      u32x4_t* dst = &lds[step % PF_STAGES][2 + pc][0];
+#pragma unroll
+      for (int i = 0; i < DC; ++i) {
+        const int slot = i * 64 + lane, h = slot / D, d = slot % D;
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(v_pages + base[pc] + (size_t)d * bs + off0[pc] + h * 8),
+                                         (lds_ptr_t)(dst + i * 64), 16, 0, 0);
+      }
     } else {
-      // slot = chunk (slot / 16) of key row (slot % 16)
-      const bf16* src = k_pages + base + (size_t)(off0 + col) * D + grp * 8;
+      // keys: slot = chunk * 32 + t holds coordinates 8 chunk .. + 7 of the key that row t of the
+      // step's two score tiles stands for (see PF_KEY_OF_ROW)
+      u32x4_t* dst = &lds[step % PF_STAGES][0][0] + wave * (DC * 64);
+      const int t = lane & 31, key = PF_KEY_OF_ROW(t >> 4, t & 15), pc = key >> 4;
+      const bf16* src = k_pages + (pc ? base[1] : base[0]) + (size_t)((pc ? off0[1] : off0[0]) + (key & 15)) * D +
+                        (wave * (2 * DC) + (lane >> 5)) * 8;
 #pragma unroll
       for (int i = 0; i < DC; ++i)
-        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + i * 32), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + i * 16), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
     }
   };
   const int nrounds = (nsteps + 1) / 2;
@@ -607,12 +623,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) sc[qt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      // The operands of a whole tile are asked from LDS before its products start, and the next
+      // tile's while they run: a product must not wait for a read issued just before it.
+      u32x4_t kraw[2][DC];
+      auto read_keys = [&](int tt, u32x4_t (&into)[DC]) {
+        // score tile tt: rows PF_KEY_OF_ROW(tt & 1, .) of step tt >> 1
+        const u32x4_t* keys = &lds[(2 * rd + (tt >> 1)) % PF_STAGES][0][0] + (tt & 1) * 16 + col;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) into[c] = keys[(c * 4 + grp) * 32];
+      };
+      read_keys(0, kraw[0]);
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) {
-        const u32x4_t* piece = &lds[(2 * rd + (tt >> 1)) % PF_STAGES][tt & 1][0];
+        if (tt + 1 < 4) read_keys(tt + 1, kraw[(tt + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);  // or the compiler moves every read down to its product
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
-          const bf16x8_t kop = __builtin_bit_cast(bf16x8_t, piece[(c * 4 + grp) * 16 + col]);
+          const bf16x8_t kop = __builtin_bit_cast(bf16x8_t, kraw[tt & 1][c]);
 #pragma unroll
           for (int qt = 0; qt < 2; ++qt)
             sc[qt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[qt][c], sc[qt][tt], 0, 0, 0);
@@ -631,7 +658,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
           for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int key = kb + 16 * tt + 4 * grp + r;
+              const int key = kb + 32 * (tt >> 1) + PF_KEY_OF_ROW(tt & 1, 4 * grp + r);
               const bool seen = key <= qpos[qt] && (window <= 0 || key > qpos[qt] - window);
               sc[qt][tt][r] = seen ? sc[qt][tt][r] : NEG_INF;
             }
@@ -671,18 +698,21 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha[qt];
       }
+      u32x4_t vraw[2][DT];
+      auto read_values = [&](int j, u32x4_t (&into)[DT]) {
+        // this lane's eight weights of step j belong to keys 8 grp .. 8 grp + 7: one 16-byte slot
+        const u32x4_t* values = &lds[(2 * rd + j) % PF_STAGES][2 + (grp >> 1)][(grp & 1) * D + col];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) into[dt] = values[dt * 16];
+      };
+      read_values(0, vraw[0]);
+      read_values(1, vraw[1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const bf16* stage_v = reinterpret_cast<const bf16*>(&lds[(2 * rd + j) % PF_STAGES][2][0]);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          bf16x8_t vop;
-#pragma unroll
-          for (int tt = 0; tt < 2; ++tt) {
-            const bf16x4_t v4 = *reinterpret_cast<const bf16x4_t*>(stage_v + tt * (PIECE * 8) + (dt * 16 + col) * 16 + 4 * grp);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = v4[r];
-          }
+          const bf16x8_t vop = __builtin_bit_cast(bf16x8_t, vraw[j][dt]);
 #pragma unroll
           for (int qt = 0; qt < 2; ++qt) o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt][j], o[qt][dt], 0, 0, 0);
         }

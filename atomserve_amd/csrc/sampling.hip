@@ -123,6 +123,7 @@ struct TopKShared {
   unsigned long long red[17];
   unsigned long long cand[SAMPLE_CAND];
   unsigned int hist[256];
+  int wave_total[4];
   unsigned int count;
   unsigned int prefix;
   unsigned int remaining;
@@ -143,14 +144,30 @@ __device__ int block_topk(const float* __restrict__ x, int V, int k, unsigned lo
       __syncthreads();
       if (mine != 0ull && (myval & mask) == prefix) atomicAdd(&sh.hist[(myval >> shift) & 255], 1u);
       __syncthreads();
-      if (tid == 0) {
-        int acc = 0, b = 255;
-        for (; b > 0; --b) {
-          if (acc + (int)sh.hist[b] >= want) break;
-          acc += sh.hist[b];
+      // The digit of the want-th largest: the bin b with (values in bins > b) < want <= (values
+      // in bins >= b).  Thread b holds bin b; the counts from a bin upwards come from a scan
+      // over the four waves that hold the 256 bins (a walk by one thread costs an LDS round
+      // trip per bin).
+      int above_incl = 0, own = 0;
+      if (tid < 256) {
+        own = (int)sh.hist[tid];
+        above_incl = own;
+        const int lane = tid & 63;
+#pragma unroll
+        for (int off = 1; off < WAVE; off <<= 1) {
+          const int o = __shfl_down(above_incl, off, WAVE);
+          if (lane + off < WAVE) above_incl += o;
         }
-        sh.prefix = prefix | ((unsigned int)b << shift);
-        sh.remaining = want - acc;
+        if (lane == 0) sh.wave_total[tid >> 6] = above_incl;
+      }
+      __syncthreads();
+      if (tid < 256) {
+        for (int w = (tid >> 6) + 1; w < 4; ++w) above_incl += sh.wave_total[w];
+        const int above = above_incl - own;  // values in higher bins
+        if (above < want && above_incl >= want) {  // exactly one bin
+          sh.prefix = prefix | ((unsigned int)tid << shift);
+          sh.remaining = want - above;
+        }
       }
       __syncthreads();
       prefix = sh.prefix;
@@ -369,7 +386,7 @@ __global__ __launch_bounds__(SPLIT_THREADS) void topk_slices_kernel(
   if (threadIdx.x == 0) counts[row * SPLIT_SLICES + slice] = found;
 }
 
-__global__ __launch_bounds__(SPLIT_THREADS) void sample_candidates_kernel(
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_candidates_kernel(
     const unsigned long long* __restrict__ cand, const int* __restrict__ counts,
     const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
     const long long* __restrict__ seeds, const int* __restrict__ counters, int* __restrict__ out) {
@@ -383,19 +400,22 @@ __global__ __launch_bounds__(SPLIT_THREADS) void sample_candidates_kernel(
   int k = effective_top_k(T, top_k[row], p_keep);
   if (T <= 0.f || p_keep <= 0.f) T = 1.f;
   k = k < 1 ? 1 : (k > SPLIT_KMAX ? SPLIT_KMAX : k);
+  __shared__ int found_in[SPLIT_SLICES];
+  if (tid < SPLIT_SLICES) found_in[tid] = counts[row * SPLIT_SLICES + tid];  // all loads at once
+  __syncthreads();
   if (tid == 0) {
     int at = 0;
-    for (int sl = 0; sl < SPLIT_SLICES; ++sl) { first[sl] = at; at += counts[row * SPLIT_SLICES + sl]; }
+    for (int sl = 0; sl < SPLIT_SLICES; ++sl) { first[sl] = at; at += found_in[sl]; }
     first[SPLIT_SLICES] = at;
   }
   __syncthreads();
   const int total = first[SPLIT_SLICES];
-  for (int sl = tid / SPLIT_KMAX; sl < SPLIT_SLICES; sl += SPLIT_THREADS / SPLIT_KMAX) {
+  for (int sl = tid / SPLIT_KMAX; sl < SPLIT_SLICES; sl += SAMPLE_THREADS / SPLIT_KMAX) {
     const int r = tid % SPLIT_KMAX, n = first[sl + 1] - first[sl];
     if (r < n) pool[first[sl] + r] = cand[((size_t)row * SPLIT_SLICES + sl) * SPLIT_KMAX + r];
   }
   __syncthreads();
-  for (int c = tid; c < total; c += SPLIT_THREADS) {
+  for (int c = tid; c < total; c += SAMPLE_THREADS) {
     const unsigned long long key = pool[c];
     int rank = 0;
     for (int j = 0; j < total; ++j) rank += pool[j] > key;
@@ -438,7 +458,7 @@ extern "C" int as_sample_split(const float* logits, int B, int V, const float* t
   topk_slices_kernel<<<dim3(B, SPLIT_SLICES), SPLIT_THREADS, 0, stream>>>(logits, V, temperature, top_k, top_p,
                                                                          (unsigned long long*)cand, counts);
   if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
-  sample_candidates_kernel<<<B, SPLIT_THREADS, 0, stream>>>((const unsigned long long*)cand, counts, temperature,
+  sample_candidates_kernel<<<B, SAMPLE_THREADS, 0, stream>>>((const unsigned long long*)cand, counts, temperature,
                                                             top_k, top_p, seeds, counters, out);
   return launch_status();
 }
