@@ -461,6 +461,12 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 // trip through LDS: v_permlane16_swap / v_permlane32_swap exchange rows of 16 lanes between
 // two registers.  With both operands equal to x, the results hold (rows 0 0 2 2, rows 1 1 3 3)
 // and (rows 0 1 0 1, rows 2 3 2 3) of x.
+// max(a, b, c) as the one instruction it is; NaN operands lose, as with fmaxf.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float quad_rows_max(float v) {
   auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
@@ -663,11 +669,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
               sc[qt][tt][r] = seen ? sc[qt][tt][r] : NEG_INF;
             }
         }
-        float mx = NEG_INF;
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
-          mx = fmaxf(mx, fmaxf(fmaxf(sc[qt][tt][0], sc[qt][tt][1]), fmaxf(sc[qt][tt][2], sc[qt][tt][3])));
-        mx = quad_rows_max(mx);
+        // sixteen scores to one in eight three-way maxima (fmaxf would first quiet every operand)
+        const float m0 = max3(sc[qt][0][0], sc[qt][0][1], sc[qt][0][2]), m1 = max3(sc[qt][0][3], sc[qt][1][0], sc[qt][1][1]);
+        const float m2 = max3(sc[qt][1][2], sc[qt][1][3], sc[qt][2][0]), m3 = max3(sc[qt][2][1], sc[qt][2][2], sc[qt][2][3]);
+        const float m4 = max3(sc[qt][3][0], sc[qt][3][1], sc[qt][3][2]);
+        const float mx = quad_rows_max(max3(max3(m0, m1, m2), max3(m3, m4, sc[qt][3][3]), NEG_INF));
         // base-2 softmax: scale and log2(e) are folded into one factor (positive, so maxima agree)
         const float mn = fmaxf(m[qt], mx * scale2);
         float rs = 0.f;
