@@ -49,7 +49,6 @@ class RequestCache:
     tables: list  # [group] -> list of page ids, position // block_size -> page (or RELEASED)
     hashes: list = field(default_factory=list)  # prefix hash of each full, computed page
     state_slot: int = -1
-    state_fresh: bool = True  # the slot holds nothing of this request yet
 
 
 class CacheManager:
@@ -120,7 +119,6 @@ class CacheManager:
                 table.extend(g.allocator.allocate(m))
         if self.state_groups and rc.state_slot < 0:
             rc.state_slot = self._free_slots.pop()
-            rc.state_fresh = True
         return True
 
     def release_behind_window(self, rc: RequestCache, num_computed: int) -> int:
@@ -151,7 +149,6 @@ class CacheManager:
         if rc.state_slot >= 0:
             self._free_slots.append(rc.state_slot)
             rc.state_slot = -1
-        rc.state_fresh = True
 
     # ---- prefix reuse (reference atomserve/scheduler.py:214-250) ------------------------
     def adopt_cached_prefix(self, rc: RequestCache, token_ids: list) -> int:

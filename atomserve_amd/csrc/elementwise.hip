@@ -155,22 +155,6 @@ extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const vo
   return launch_status();
 }
 
-// ---- residual sum alone (the last layer's pending delta, when no norm follows) ----
-template <typename O>
-__global__ void add_delta_kernel(float* __restrict__ x, const O* __restrict__ delta, size_t count) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
-    x[i] += to_f32(delta[i]);
-}
-
-extern "C" int as_add_delta(float* x, const void* delta, int delta_dtype, long count, hipStream_t stream) {
-  if (count <= 0) return AS_OK;
-  const int blocks = (int)((count + 255) / 256 > 4096 ? 4096 : (count + 255) / 256);
-  if (delta_dtype == DT_F32) add_delta_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)count);
-  else if (delta_dtype == DT_BF16) add_delta_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (size_t)count);
-  else return AS_BAD_DTYPE;
-  return launch_status();
-}
-
 // ---- rotary table -------------------------------------------------------------------
 // cs[t, i] = (cos, sin)(positions[t] * inv_freq[i]), i < half.  The product and the
 // range reduction are done in fp64 so that large positions keep fp32-exact angles;

@@ -39,11 +39,7 @@ def slot_of(block_table: list, position: int, block_size: int) -> int:
     return block_table[position // block_size] * block_size + position % block_size
 
 
-class _View:
-    pass
-
-
-class PagedLayerView(_View):
+class PagedLayerView:
     """What an attention mixer sees of its cache in one step."""
 
     __slots__ = ("k_pages", "v_pages", "slots", "block_tables", "writes", "block_size")
@@ -53,7 +49,7 @@ class PagedLayerView(_View):
         self.writes, self.block_size = writes, block_size
 
 
-class StateLayerView(_View):
+class StateLayerView:
     """What a mixer with fixed-size state sees: its state table and each row's slot."""
 
     __slots__ = ("state", "row_slots", "writes")

@@ -65,13 +65,6 @@ def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True) -> None:
          _DT[out.dtype], n_out, n, int(bool(update_x)), _stream())  # fmt: skip
 
 
-def add_delta(x, delta) -> None:
-    """x += delta (x fp32, delta fp32|bf16, same shape)."""
-    _check(x, "x", F32)
-    _check(delta, "delta", (F32, BF16), tuple(x.shape))
-    call("as_add_delta", _ptr(x), _ptr(delta), _DT[delta.dtype], x.numel(), _stream())
-
-
 def rope_table(positions, inv_freq, out) -> None:
     """out[t, i] = (cos, sin)(positions[t] * inv_freq[i]); inv_freq fp64 [R/2], out fp32 [T, R/2, 2]."""
     _check(positions, "positions", I32, (None,))

@@ -33,6 +33,7 @@ def write_random_model(path: str, config, seed: int, dtype=torch.bfloat16, std: 
     from atomserve_amd.config.registry import architecture_for
 
     raw = config.to_dict()
+    raw["torch_dtype"] = str(dtype).replace("torch.", "")  # what the file holds
     arch = architecture_for(raw)
     os.makedirs(path, exist_ok=True)
     tensors = random_checkpoint(arch, config, seed, dtype=dtype, std=std, gain_std=gain_std)

@@ -40,6 +40,7 @@ def parse_args():
     p.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     p.add_argument("--points", default="1,64", help="other decode batch sizes to measure (fewer steps each)")
     p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--no-calibration", action="store_true", help="skip the library copy and matmul probes")
     p.add_argument("--greedy", action="store_true", help="greedy instead of the default sampling settings")
     return p.parse_args()
 
@@ -47,6 +48,29 @@ def parse_args():
 def prompt(b: int, n: int, vocab: int) -> list:
     """Distinct synthetic prompts (reference bench/engine.py:90-92)."""
     return [(1000 + 37 * b + i) % (vocab - 1000) for i in range(n)]
+
+
+def calibrate(device) -> dict:
+    """What this GPU delivers to plain library calls, to read the roofline fractions against: a
+    1 GiB device copy (bytes read plus written per second) and an 8192^3 bf16 matrix product."""
+    import torch
+
+    def timed(fn, n=5):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    x = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    y = torch.empty_like(x)
+    copy = 2 * x.numel() / timed(lambda: y.copy_(x))
+    a = torch.randn(8192, 8192, device=device).to(torch.bfloat16)
+    b = torch.randn(8192, 8192, device=device).to(torch.bfloat16)
+    matmul = 2 * 8192**3 / timed(lambda: torch.mm(a, b.t()))
+    return {"copy_GBps": round(copy / 1e9, 1), "matmul_bf16_TFLOPs": round(matmul / 1e12, 1)}
 
 
 def main() -> int:
@@ -67,6 +91,7 @@ def main() -> int:
 
     device = "cuda:0"
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    calibration = None if args.no_calibration else calibrate(device)
     config = Qwen3Config(**{**SIZES, "num_layers": args.layers})
     arch = architecture_for(config.to_dict())
     model = DecoderModel(arch.build_plan(config), dtype, device)
@@ -143,7 +168,7 @@ def main() -> int:
     achieved = step_bytes / (ms * 1e-3)
 
     line = {
-        "metric": "decode tok/s at batch 8, 2048-token contexts (Qwen3-8B sizes, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, {args.context}-token contexts (Qwen3-8B sizes, random weights)",
         "value": round(tps, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -168,6 +193,8 @@ def main() -> int:
     }
     if result_prefill:
         line["prefill"] = result_prefill
+    if calibration:
+        line["calibration"] = calibration
     print(json.dumps(line))
     return 0
 
