@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
   const int G = H / KV;
   const int HC = (G + GT - 1) / GT;
   const int item = blockIdx.x, kvh = blockIdx.y / HC, hc = blockIdx.y % HC, part = blockIdx.z;
-  const int t = items[item];
+  const int t = items ? items[item] : item;  // null: every token, in order
   const int pos = positions[t];
   const int ctx = pos + 1;
   const int lo = window > 0 ? max(0, ctx - window) : 0;
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void attn_single_query_kernel(
   const int nsub = 64 / lpk;  // keys in flight per wave
   const int sub = lane / lpk, j = lane % lpk;
   const bool active = j * CH < D;
-  const int* table = block_tables + (size_t)tok_row[t] * table_width;
+  const int* table = block_tables + (size_t)(tok_row ? tok_row[t] : t) * table_width;  // null: token t is row t
 
   float qr[GT][CH];
 #pragma unroll
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(const int* __restrict_
     den += (mp == NEG_INF) ? 0.f : part_l[base + p] * fexp<T>(mp - mx);
   }
   const float inv = 1.0f / den;
-  const int t = items[item];
+  const int t = items ? items[item] : item;  // null: every token, in order
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float num = 0.f;
 #pragma unroll 4
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   extern __shared__ float smem[];          // [4][16] m, [4][16] l, [4][D][G] acc
   const int G = H / KV;
   const int item = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
-  const int t = items[item];
+  const int t = items ? items[item] : item;  // null: every token, in order
   const int pos = positions[t];
   const int ctx = pos + 1;
   const int lo = window > 0 ? max(0, ctx - window) : 0;
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       part_acc[(((size_t)item * H + h0 + idx / D) * P + part) * D + idx % D] = 0.f;
     return;
   }
-  const int* table = block_tables + (size_t)tok_row[t] * table_width;
+  const int* table = block_tables + (size_t)(tok_row ? tok_row[t] : t) * table_width;  // null: token t is row t
 
   bf16x8_t qop[DC];
   {

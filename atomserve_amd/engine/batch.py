@@ -175,6 +175,7 @@ class StepBatch:
         self._staging, self._widths, self._vocab = staging, widths, vocab_size
 
         self.num_tokens, self.num_rows = T, R
+        self.decode_only = all(len(row.tokens) == 1 for row in rows)  # token t is row t
         self.token_ids, self.positions, self.tok_row = parts["token_ids"], parts["positions"], parts["tok_row"]
         self.logits_rows, self.num_logits = parts["logits_rows"], len(want)
         self.all_tokens = parts["all_tokens"]

@@ -129,19 +129,24 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
     of 32, groups of up to 16 heads and pages of a multiple of 16 tokens runs on the matrix cores;
     everything else (and all of fp32) on the general kernel.
 
-    q, out [T, H, D]; items [N] int32: the tokens (rows of q) to process; positions, tok_row [T]
-    int32; block_tables [R, W] int32; max_context: host bound on positions[items] + 1."""
+    q, out [T, H, D]; items [N] int32: the tokens (rows of q) to process, None for all of them in
+    order; positions, tok_row [T] int32 (tok_row None: token t belongs to row t, a decode step);
+    block_tables [R, W] int32; max_context: host bound on positions[items] + 1."""
     _check(q, "q", (F32, BF16), (None, None, None))
     T, H, D = q.shape
     _check(out, "out", q.dtype, (T, H, D))
     _check(k_pages, "k_pages", q.dtype, (None, None, None, D))
     _, KV, bs, _ = k_pages.shape
     _check(v_pages, "v_pages", q.dtype, (k_pages.shape[0], KV, D, bs))
-    _check(items, "items", I32, (None,))
+    if items is not None:
+        _check(items, "items", I32, (None,))
     _check(positions, "positions", I32, (T,))
-    _check(tok_row, "tok_row", I32, (T,))
+    if tok_row is not None:
+        _check(tok_row, "tok_row", I32, (T,))
     _check(block_tables, "block_tables", I32, (None, None))
-    N = items.shape[0]
+    if tok_row is None and block_tables.shape[0] < T:
+        raise KernelError(f"attention: {T} tokens that are their own rows need as many block tables")
+    N = T if items is None else items.shape[0]
     if N == 0:
         return
     chunk = 4 if q.dtype == F32 else 8

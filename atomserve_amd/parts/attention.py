@@ -74,6 +74,10 @@ class Attention(Mixer):
         s = self.spec
         # fp32, and shapes the prefill kernel does not take: every token is a single query.
         # Otherwise short rows are single queries and long rows go through the prefill kernel.
+        if step.decode_only:  # token t is row t: the kernels need no maps from one to the other
+            ops.attn_single_query(q, cache.k_pages, cache.v_pages, None, step.positions, None, cache.block_tables,
+                                  out, s.scale, s.window, step.max_context)  # fmt: skip
+            return
         if not ops.attn_prefill_supported(self.env.dtype, s.head_dim, cache.block_size):
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
                                   cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip

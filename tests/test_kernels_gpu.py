@@ -341,6 +341,24 @@ def test_attention_window_edge(ops, window, dtype, bs):
     assert torch.allclose(out.float(), ref, atol=1e-5 if dtype == F32 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_attention_of_a_decode_step_needs_no_maps(ops, dtype):
+    """Every token is a row of its own: without the token list and the token-to-row map the
+    kernels do exactly what they do with the identity maps."""
+    H, KV, D, bs = 8, 2, 64, 16
+    lens = [1, 37, 300, 513]
+    q, k_pages, v_pages, tables, positions = paged_case(dtype, H, KV, D, bs, lens, seed=7)
+    ident = i32(list(range(4)))
+    a = torch.zeros(4, H, D, dtype=dtype, device=DEV)
+    b = torch.zeros_like(a)
+    for part in (None, 64):
+        ops.attn_single_query(q, k_pages, v_pages, ident, positions, ident, tables, a, D**-0.5, 0, max(lens), part)
+        ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables, b, D**-0.5, 0, max(lens), part)
+        assert torch.equal(a, b)
+    with pytest.raises(ops.KernelError):
+        ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables[:3], b, D**-0.5, 0, max(lens))
+
+
 def test_attention_serves_only_the_listed_tokens(ops):
     """Items select tokens; several tokens of one request share a table and see keys up to
     their own position only."""
