@@ -399,6 +399,21 @@ def test_attention_prefill(ops, H, KV, D, bs, window):
     assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), (out.float() - ref).abs().max()
 
 
+def test_attention_prefill_of_a_long_prompt_in_one_step(ops):
+    """4,500 tokens at once after a prefix of 700: many more work items than the GPU holds at a
+    time, in the order the engine gives them (most keys first), hundreds of rounds per item."""
+    H, KV, D, bs, start, n = 8, 2, 128, 16, 700, 4500
+    torch.manual_seed(15)
+    _, k_pages, v_pages, tables, _ = paged_case(BF16, H, KV, D, bs, [start + n], seed=9, k_scale=2.0 / math.sqrt(D / 16))
+    q = torch.randn(n, H, D, device=DEV).to(BF16)
+    tiles = sorted(([q0, min(64, n - q0), 0, start + q0] for q0 in range(0, n, 64)), key=lambda t: -(t[3] + t[1]))
+    out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
+    ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, 0, start + n)
+    check = list(range(0, n, 97)) + [n - 1]
+    ref = pk.paged_attention(q, k_pages, v_pages, i32(check), i32(list(range(start, start + n))), i32([0] * n), tables, D**-0.5)
+    assert torch.allclose(out[check].float(), ref[check], atol=2e-2, rtol=2e-2), (out[check].float() - ref[check]).abs().max()
+
+
 def test_attention_prefill_sees_a_far_key_and_not_the_future(ops):
     H, KV, D, bs, n = 4, 2, 64, 16, 700
     for far in (0, 17, 255, 256, 640):

@@ -82,6 +82,21 @@ def test_first_tokens_and_long_decoding(setup, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_across_the_context_bound_of_a_captured_graph(dtype, tmp_path):
+    """Replayed decode steps are captured for contexts up to a multiple of 1,024 tokens; a request
+    that decodes from 1,009 to 1,040 tokens passes from one captured step to the next."""
+    raw = dict(TINY["A"], max_position_embeddings=2048)
+    weights = plain_random_weights(raw, seed=47, std=0.2, gain_std=0.2)
+    path = write_model_dir(str(tmp_path / "long"), raw, weights, torch.bfloat16)
+    ids = rc.random_ids(raw["vocab_size"], 1040, seed=6)
+    steps = rc.prefill_then_decode("a", ids)
+    replay = make_replay(path, dtype, rc.live_token_bound(steps))
+    worst, scale, rows = rc.run_and_compare(replay, steps, {"a": ids}, raw, weights, {})
+    assert rows == 33 and len(replay.runner.decode_graphs.graphs) == 2
+    check(worst, scale, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("num_requests", [3, 13, 40])
 def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
     """Decode steps replayed as captured graphs against the same steps launched kernel by kernel:
