@@ -104,10 +104,67 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, floatx4 v, int
   for (int i = 0; i < valid; ++i) p[i] = (bf16)v[i];
 }
 
-template <int S, int MT, int SK_WAVES, typename OutT>
+// What a few-rows product carries along when the residual sum and the RMSNorm around it are
+// folded into the products of a decode step (a pre-norm layer: x += part(norm(x))):
+//
+//   producer (LINK): out is the fp32 stream x[M, N] and receives the bf16-rounded product on
+//     top; the same lanes then write scaled[m, n] = bf16(x * gain[n]), the input of the next
+//     product without its 1/rms factor, and ssq[m, strip] = the sum of x^2 over the strip's 16
+//     columns.  Every element belongs to one lane of one workgroup: no races, a fixed order.
+//   consumer (SCALED): a is such a `scaled`; 1/rms of each row comes from the row's sums of
+//     squares (added in a fixed order, in fp32) and multiplies the product's fp32 sums before
+//     anything else happens to them.  x * gain / rms is rounded to bf16 once in the RMSNorm
+//     kernel and x * gain once here: the same precision, not the same bits.
+struct NormLink {
+  const float* ssq_in;  // SCALED: [M, strips_in]
+  int strips_in;
+  float eps;
+  const float* gain;    // LINK: [N], the gains of the norm that follows
+  bf16* scaled;         // LINK: [M, N]
+  float* ssq_out;       // LINK: [M, strips of this product]
+};
+
+// The LINK epilogue for the lane that holds columns n .. n+3 of row m (sum: the product's fp32
+// sums).  All 64 lanes of the wave call it together.
+__device__ __forceinline__ void link_epilogue(const NormLink& link, float* x, floatx4 sum, int m, int n, int M, int N,
+                                              int strip, int nstrips) {
+  float ss = 0.f;
+  if (m < M && n < N) {
+    const int valid = min(4, N - n);
+    float* xp = x + (size_t)m * N + n;
+    bf16* sp = link.scaled + (size_t)m * N + n;
+    if (valid == 4) {  // N % 4 == 0 here or this is not the last group: 16-byte aligned
+      floatx4 v = *reinterpret_cast<floatx4*>(xp);
+      const floatx4 g = *reinterpret_cast<const floatx4*>(link.gain + n);
+      typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+      bf16x4 sc;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] += (float)(bf16)sum[r];
+        sc[r] = (bf16)(v[r] * g[r]);
+        ss += v[r] * v[r];
+      }
+      *reinterpret_cast<floatx4*>(xp) = v;
+      *reinterpret_cast<bf16x4*>(sp) = sc;
+    } else {
+      for (int r = 0; r < valid; ++r) {
+        const float v = xp[r] + (float)(bf16)sum[r];
+        xp[r] = v;
+        sp[r] = (bf16)(v * link.gain[n + r]);
+        ss += v * v;
+      }
+    }
+  }
+  ss += __shfl_xor(ss, 16, 64);  // the four lanes that hold the strip's 16 columns of row m
+  ss += __shfl_xor(ss, 32, 64);
+  if ((threadIdx.x & 63) < 16 && m < M) link.ssq_out[(size_t)m * nstrips + strip] = ss;
+}
+
+template <int S, int MT, int SK_WAVES, typename OutT, bool LINK = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(const bf16* __restrict__ a,
                                                                         const bf16* __restrict__ w,
-                                                                        OutT* __restrict__ out, int M, int N, int K) {
+                                                                        OutT* __restrict__ out, int M, int N, int K,
+                                                                        NormLink link = NormLink{}) {
   extern __shared__ floatx4 red[];  // [SK_WAVES][S * MT][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
@@ -199,7 +256,12 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(const b
     for (int wv_ = 1; wv_ < SK_WAVES; ++wv_) sum += red[wv_ * (S * MT * 64) + e];
     const int l = e & 63, tile = e >> 6, s = tile / MT, mt = tile % MT;
     const int m = mt * 16 + (l & 15), n = n0 + s * 16 + 4 * (l >> 4);
-    if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
+    if constexpr (LINK) {
+      static_assert(!LINK || (S == 1 && MT == 1), "one strip, one wave of lanes");
+      link_epilogue(link, reinterpret_cast<float*>(out), sum, m, n, M, N, blockIdx.x, gridDim.x);
+    } else {
+      if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
+    }
   }
 }
 
@@ -239,14 +301,17 @@ template <typename OutT> __device__ __forceinline__ float rounded(float v);
 template <> __device__ __forceinline__ float rounded<float>(float v) { return v; }
 template <> __device__ __forceinline__ float rounded<bf16>(float v) { return (float)(bf16)v; }
 
-template <int NST, bool MASKED, bool GATED, typename OutT>
+template <int NST, bool MASKED, bool GATED, typename OutT, bool SCALED = false, bool LINK = false>
 __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(const bf16* __restrict__ a,
                                                                                const bf16* __restrict__ w,
                                                                                OutT* __restrict__ out, int M, int N,
-                                                                               int K, int nstrips) {
+                                                                               int K, int nstrips,
+                                                                               NormLink link = NormLink{}) {
   static_assert(NST % 2 == 0, "a wave's slice is handled in two halves");
+  static_assert(!LINK || (!GATED && !SCALED && sizeof(OutT) == 4), "the stream is fp32 and takes a plain product");
   constexpr int H = NST / 2;
   __shared__ floatx4 red[2][PIPE_WAVES * 64];
+  __shared__ float inv_rms[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
   const int kbase = wave * NST * 64 + lg * 16;  // this lane's first k; step u adds 64 u
@@ -281,6 +346,16 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
       av[u][1] = PIPE_VALID(u, 1) ? *reinterpret_cast<const bf16x8*>(arow + u * 64 + 8) : zero;
     }
   }
+  if constexpr (SCALED) {
+    // 1 / rms of the 16 rows, 32 threads a row; published by the first strip's barrier
+    const int row = threadIdx.x >> 5, j0 = threadIdx.x & 31;
+    float ss = 0.f;
+    if (row < M)
+      for (int j = j0; j < link.strips_in; j += 32) ss += link.ssq_in[(size_t)row * link.strips_in + j];
+#pragma unroll
+    for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off, 64);
+    if (j0 == 0) inv_rms[row] = row < M ? 1.0f / sqrtf(ss / (float)K + link.eps) : 0.f;
+  }
   int buf = 0, turn = 0;
   floatx4 gate = {0.f, 0.f, 0.f, 0.f};
   for (;;) {
@@ -299,7 +374,11 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
       floatx4 sum = red[buf][lane];
 #pragma unroll
       for (int x = 1; x < PIPE_WAVES; ++x) sum += red[buf][x * 64 + lane];
-      if (GATED && !up) {
+      if constexpr (SCALED) sum *= inv_rms[lr];
+      const int m = lr, n = strip * 16 + 4 * lg;
+      if constexpr (LINK) {
+        link_epilogue(link, reinterpret_cast<float*>(out), sum, m, n, M, N, strip, nstrips);
+      } else if (GATED && !up) {
         gate = sum;
       } else {
         if (GATED) {
@@ -309,7 +388,6 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
             sum[r] = g / (1.0f + expf(-g)) * rounded<OutT>(sum[r]);
           }
         }
-        const int m = lr, n = strip * 16 + 4 * lg;
         if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
       }
     }
@@ -327,36 +405,30 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
 #undef PIPE_MATH
 }
 
-template <int NST, bool GATED>
-static int launch_pipe(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
+template <int NST, bool GATED, typename OutT, bool SCALED, bool LINK>
+static int launch_pipe(const void* a, const void* w, void* out, int M, int N, int K, const NormLink& link,
                        hipStream_t stream) {
   const int nstrips = (N + 15) / 16;
   const int blocks = min(nstrips, compute_units());
-  const bool exact = K == 64 * PIPE_WAVES * NST;
-#define PIPE_GO(MASKED, OutT)                                                                        \
-  gemm_bf16_skinny_pipe_kernel<NST, MASKED, GATED, OutT><<<blocks, PIPE_WAVES * 64, 0, stream>>>(    \
-      (const bf16*)a, (const bf16*)w, (OutT*)out, M, N, K, nstrips)
-  if (out_dtype == DT_BF16) {
-    if (exact) PIPE_GO(false, bf16); else PIPE_GO(true, bf16);
-  } else if (out_dtype == DT_F32) {
-    if (exact) PIPE_GO(false, float); else PIPE_GO(true, float);
-  } else {
-    return AS_BAD_DTYPE;
-  }
-#undef PIPE_GO
+  if (K == 64 * PIPE_WAVES * NST)
+    gemm_bf16_skinny_pipe_kernel<NST, false, GATED, OutT, SCALED, LINK><<<blocks, PIPE_WAVES * 64, 0, stream>>>(
+        (const bf16*)a, (const bf16*)w, (OutT*)out, M, N, K, nstrips, link);
+  else
+    gemm_bf16_skinny_pipe_kernel<NST, true, GATED, OutT, SCALED, LINK><<<blocks, PIPE_WAVES * 64, 0, stream>>>(
+        (const bf16*)a, (const bf16*)w, (OutT*)out, M, N, K, nstrips, link);
   return launch_status();
 }
 
-template <bool GATED>
-static int dispatch_pipe(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
-                         hipStream_t stream) {
+template <bool GATED, typename OutT, bool SCALED = false, bool LINK = false>
+static int dispatch_pipe(const void* a, const void* w, void* out, int M, int N, int K, hipStream_t stream,
+                         const NormLink& link = NormLink{}) {
   switch (2 * ((K + 128 * PIPE_WAVES - 1) / (128 * PIPE_WAVES))) {
-    case 2: return launch_pipe<2, GATED>(a, w, out, out_dtype, M, N, K, stream);
-    case 4: return launch_pipe<4, GATED>(a, w, out, out_dtype, M, N, K, stream);
-    case 6: return launch_pipe<6, GATED>(a, w, out, out_dtype, M, N, K, stream);
-    case 8: return launch_pipe<8, GATED>(a, w, out, out_dtype, M, N, K, stream);
-    case 10: return launch_pipe<10, GATED>(a, w, out, out_dtype, M, N, K, stream);
-    case 12: return launch_pipe<12, GATED>(a, w, out, out_dtype, M, N, K, stream);
+    case 2: return launch_pipe<2, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
+    case 4: return launch_pipe<4, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
+    case 6: return launch_pipe<6, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
+    case 8: return launch_pipe<8, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
+    case 10: return launch_pipe<10, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
+    case 12: return launch_pipe<12, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
   }
   return AS_BAD_SHAPE;
 }
@@ -364,14 +436,45 @@ static int dispatch_pipe(const void* a, const void* w, void* out, int out_dtype,
 // Whether the persistent kernel takes a product of these sizes.
 static bool pipe_fits(int M, int K) { return M <= 16 && K <= 64 * PIPE_WAVES * PIPE_MAX_NST; }
 
-// out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for w[2N, K], both products rounded to the
-// output type before the activation.  Only sizes of the persistent kernel; AS_BAD_SHAPE
+// out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for w[2N, K] in bf16, both products rounded
+// to bf16 before the activation.  Only sizes of the persistent kernel; AS_BAD_SHAPE
 // otherwise, and the caller runs the product and the activation kernel instead.
-extern "C" int as_gemm_bf16_gated(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
+extern "C" int as_gemm_bf16_gated(const void* a, const void* w, void* out, int M, int N, int K,
                                   hipStream_t stream) {
   if (M <= 0) return AS_OK;
   if (N <= 0 || K <= 0 || (K & 7) || !pipe_fits(M, K)) return AS_BAD_SHAPE;
-  return dispatch_pipe<true>(a, w, out, out_dtype, M, N, K, stream);
+  return dispatch_pipe<true, bf16>(a, w, out, M, N, K, stream);
+}
+
+// The producer of a NormLink: x[M, N] (fp32) += bf16(a @ w^T); scaled[M, N] = bf16(x * gain);
+// ssq[M, ceil(N / 16)] = sums of x^2 per 16 columns.  M <= 16, K % 8 == 0, N % 4 == 0; a K beyond
+// the persistent kernel goes through the streaming one.
+extern "C" int as_gemm_bf16_link(const void* a, const void* w, float* x, const float* gain, void* scaled,
+                                 float* ssq, int M, int N, int K, hipStream_t stream) {
+  if (M <= 0) return AS_OK;
+  if (M > 16 || N <= 0 || K <= 0 || (K & 7) || (N & 3) || !gain || !scaled || !ssq) return AS_BAD_SHAPE;
+  const NormLink link{nullptr, 0, 0.f, gain, (bf16*)scaled, ssq};
+  if (pipe_fits(M, K)) return dispatch_pipe<false, float, false, true>(a, w, x, M, N, K, stream, link);
+  const int blocks = (N + 15) / 16;
+  if (blocks < 512)
+    gemm_bf16_skinny_kernel<1, 1, 16, float, true><<<blocks, 16 * 64, sizeof(floatx4) * 16 * 64, stream>>>(
+        (const bf16*)a, (const bf16*)w, x, M, N, K, link);
+  else
+    gemm_bf16_skinny_kernel<1, 1, 8, float, true><<<blocks, 8 * 64, sizeof(floatx4) * 8 * 64, stream>>>(
+        (const bf16*)a, (const bf16*)w, x, M, N, K, link);
+  return launch_status();
+}
+
+// The consumer of a NormLink: out[M, N] (bf16) = (scaled @ w^T) / rms(x) with rms from
+// ssq[M, strips_in] (strips_in = ceil(K / 16)) and eps; gated != 0: the gated product of that.
+// Only sizes of the persistent kernel.
+extern "C" int as_gemm_bf16_scaled(const void* scaled, const float* ssq, int strips_in, float eps, const void* w,
+                                   void* out, int M, int N, int K, int gated, hipStream_t stream) {
+  if (M <= 0) return AS_OK;
+  if (N <= 0 || K <= 0 || (K & 7) || !pipe_fits(M, K) || !ssq || strips_in != (K + 15) / 16) return AS_BAD_SHAPE;
+  const NormLink link{ssq, strips_in, eps, nullptr, nullptr, nullptr};
+  return gated ? dispatch_pipe<true, bf16, true, false>(scaled, w, out, M, N, K, stream, link)
+               : dispatch_pipe<false, bf16, true, false>(scaled, w, out, M, N, K, stream, link);
 }
 
 // strips: rows of w per workgroup / 16 in the streaming kernel (1, 2 or 4); 0 lets this
@@ -385,7 +488,11 @@ extern "C" int as_gemm_bf16_skinny(const void* a, const void* w, void* out, int 
   if (M > 64 || N <= 0 || K <= 0 || (K & 7)) return AS_BAD_SHAPE;
   const int MT = (M + 15) / 16;
   if (strips == 0 || strips == -1) {
-    if (pipe_fits(M, K)) return dispatch_pipe<false>(a, w, out, out_dtype, M, N, K, stream);
+    if (pipe_fits(M, K)) {
+      if (out_dtype == DT_BF16) return dispatch_pipe<false, bf16>(a, w, out, M, N, K, stream);
+      if (out_dtype == DT_F32) return dispatch_pipe<false, float>(a, w, out, M, N, K, stream);
+      return AS_BAD_DTYPE;
+    }
     if (strips == -1) return AS_BAD_SHAPE;
   }
   int S = strips;

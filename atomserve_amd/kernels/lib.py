@@ -27,7 +27,9 @@ SIGNATURES = {
     "as_attn_prefill_mfma": ("attention", [P, P, P, P, I, P, I, P, I, I, I, I, F, I, P]),
     "as_gemm_f32": ("gemm", [P, P, P, I, I, I, P]),
     "as_gemm_bf16_skinny": ("gemm", [P, P, P, I, I, I, I, I, P]),
-    "as_gemm_bf16_gated": ("gemm", [P, P, P, I, I, I, I, P]),
+    "as_gemm_bf16_gated": ("gemm", [P, P, P, I, I, I, P]),
+    "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, I, I, I, P]),
+    "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, I, I, I, I, P]),
     "as_argmax": ("sampling", [P, P, I, I, P]),
     "as_sample": ("sampling", [P, I, I, P, P, P, P, P, P, P]),
     "as_sample_split": ("sampling", [P, I, I, P, P, P, P, P, P, P, P, P]),

@@ -261,11 +261,52 @@ def gemm_silu_mul(a, w, out) -> None:
     if M == 0:
         return
     if a.dtype == BF16 and M <= SKINNY_MAX_ROWS and K % 8 == 0 and K <= GATED_MAX_K:
-        call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, inter, K, _stream())
+        call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), M, inter, K, _stream())
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
     gemm(a, w, gate_up)
     silu_mul(gate_up, out)
+
+
+def gemm_link_supported(rows: int, n_out: int, k: int, dtype) -> bool:
+    """Whether `gemm_link` and, for its result, `gemm_scaled` exist: bf16, few rows, widths the
+    kernels take (n_out is the width of the stream, which is the next product's input)."""
+    return (dtype == BF16 and 0 < rows <= SKINNY_MAX_ROWS and k % 8 == 0 and n_out % 8 == 0
+            and n_out <= GATED_MAX_K)  # fmt: skip
+
+
+def gemm_link(a, w, x, gain, scaled, ssq) -> None:
+    """The last product of a part of a pre-norm layer with the residual sum and the first half of
+    the next RMSNorm: x[M, N] (fp32) += bf16(a @ w^T); scaled[M, N] = bf16(x * gain), the next
+    product's input without its 1/rms factor; ssq[M, ceil(N / 16)] = sums of x^2 per 16 columns.
+    a, w bf16; gain fp32 [N]."""
+    _check(a, "a", BF16, (None, None))
+    M, K = a.shape
+    _check(w, "w", BF16, (None, K))
+    N = w.shape[0]
+    if not gemm_link_supported(M, N, K, a.dtype):
+        raise KernelError(f"gemm_link: {M} rows, {K} -> {N} have no fused kernel")
+    _check(x, "x", F32, (M, N))
+    _check(gain, "gain", F32, (N,))
+    _check(scaled, "scaled", BF16, (M, N))
+    _check(ssq, "ssq", F32, (M, -(-N // 16)))
+    call("as_gemm_bf16_link", _ptr(a), _ptr(w), _ptr(x), _ptr(gain), _ptr(scaled), _ptr(ssq), M, N, K, _stream())
+
+
+def gemm_scaled(scaled, ssq, eps, w, out, gated=False) -> None:
+    """The first product of the part that follows a `gemm_link`: out = (scaled @ w^T) / rms with
+    rms^2 = sum(ssq) / K + eps per row (gated: silu of the first half of w's rows times the
+    second half, both scaled and rounded to bf16 first).  scaled [M, K], w, out bf16."""
+    _check(scaled, "scaled", BF16, (None, None))
+    M, K = scaled.shape
+    _check(ssq, "ssq", F32, (M, -(-K // 16)))
+    _check(out, "out", BF16, (M, None))
+    N = out.shape[1]
+    _check(w, "w", BF16, (2 * N if gated else N, K))
+    if not gemm_link_supported(M, K, 8, BF16):
+        raise KernelError(f"gemm_scaled: {M} rows of width {K} have no fused kernel")
+    call("as_gemm_bf16_scaled", _ptr(scaled), _ptr(ssq), ssq.shape[1], float(eps), _ptr(w), _ptr(out), M, N, K,
+         int(bool(gated)), _stream())  # fmt: skip
 
 
 SAMPLE_MAX_TOP_K = 1024

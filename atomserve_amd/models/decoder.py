@@ -83,7 +83,11 @@ class DecoderModel:
         ops.embed_gather(self.embed_weight, step.token_ids, x)
         delta = None
         for i, r in enumerate(p.run):
-            delta = self.blocks[r.layer].forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes))
+            # the norm that the run after this one starts with: this run's last product may add
+            # into x and leave that norm pending instead of handing over a delta
+            follows = self.blocks[p.run[i + 1].layer].first_norm() if i + 1 < len(p.run) else None
+            delta = self.blocks[r.layer].forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes),
+                                                 next_norm=follows)  # fmt: skip
         n = step.num_logits
         logits = torch.empty((n, p.vocab_size), dtype=torch.float32, device=dev)
         if n:

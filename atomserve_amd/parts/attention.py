@@ -12,7 +12,7 @@ run's cache computes q alone and stores nothing.
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import Mixer, PagedCacheRequest, WeightDecl, build, register
+from atomserve_amd.parts.base import Mixer, PagedCacheRequest, PendingNorm, WeightDecl, build, register
 
 # Rows with at most this many new tokens are attended as that many single queries
 # (reference atomserve/runner.py:31-34); longer rows go through the prefill kernel.
@@ -20,6 +20,9 @@ SHORT_ROW = 8
 
 
 class Attention(Mixer):
+    takes_pending_norm = True
+    adds_to_residual = True
+
     def __init__(self, spec, env):
         super().__init__(spec, env)
         s = spec
@@ -49,24 +52,33 @@ class Attention(Mixer):
         s = self.spec
         return PagedCacheRequest(s.num_kv_heads, s.head_dim, s.window)
 
-    def forward(self, h, step, cache):
-        """h [T, hidden] compute dtype -> [T, hidden].  cache: a PagedLayerView (pages of this
-        run's cache, its group's slots and block tables for this step, whether to store)."""
+    def forward(self, h, step, cache, residual=None, next_norm=None):
+        """h [T, hidden] compute dtype (or the norm left pending on the stream) -> [T, hidden], or the
+        pending `next_norm` after adding the output into `residual`.  cache: a PagedLayerView (pages
+        of this run's cache, its group's slots and block tables for this step, whether to store)."""
         s, env = self.spec, self.env
-        T = h.shape[0]
+        pending = isinstance(h, PendingNorm)
+        T, device = (h.x.shape[0], h.x.device) if pending else (h.shape[0], h.device)
         H, KV, D = s.num_heads, s.num_kv_heads, s.head_dim
-        qkv = torch.empty((T, (H + 2 * KV) * D), dtype=env.dtype, device=h.device)
-        ops.gemm(h, self.qkv_weight, qkv)
-        q = torch.empty((T, H, D), dtype=env.dtype, device=h.device)
+        qkv = torch.empty((T, (H + 2 * KV) * D), dtype=env.dtype, device=device)
+        if pending:
+            h.gemm(self.qkv_weight, qkv)
+        else:
+            ops.gemm(h, self.qkv_weight, qkv)
+        q = torch.empty((T, H, D), dtype=env.dtype, device=device)
         cos_sin = self.position.prepare(step) if self.position is not None else None
         eps = s.qk_norm.eps if s.qk_norm is not None else 0.0
         ops.qk_norm_rope_store(
             qkv.view(T, H + 2 * KV, D), self.q_norm_weight, self.k_norm_weight, cos_sin, cache.slots, q,
             cache.k_pages, cache.v_pages, H, KV, eps, store_kv=cache.writes,
         )  # fmt: skip
-        out = torch.empty((T, H, D), dtype=env.dtype, device=h.device)
+        out = torch.empty((T, H, D), dtype=env.dtype, device=device)
         self.attend(q, out, step, cache)
-        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=h.device)
+        if residual is not None and next_norm is not None:
+            link = next_norm.absorb(out.view(T, H * D), self.o_weight, residual)
+            if link is not None:
+                return link
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=device)
         ops.gemm(out.view(T, H * D), self.o_weight, y)
         return y
 

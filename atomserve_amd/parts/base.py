@@ -80,7 +80,37 @@ class BuildEnv:
     device: torch.device
 
 
+class PendingNorm:
+    """A norm of the fp32 stream `x` whose last step is still due: the part before has added its
+    output into `x` and left what the norm's consumer needs to finish the norm inside its first
+    matrix product (`gemm`, `gemm_silu_mul`).  `rows()` runs the norm's own kernel on `x` for a
+    consumer that wants the normalised rows themselves."""
+
+    def __init__(self, norm: "Norm", x: torch.Tensor):
+        self.norm = norm
+        self.x = x
+
+    def rows(self) -> torch.Tensor:
+        return self.norm.forward(self.x)
+
+    def gemm(self, w: torch.Tensor, out: torch.Tensor) -> None:
+        """out = norm(x) @ w^T"""
+        raise NotImplementedError
+
+    def gemm_silu_mul(self, w: torch.Tensor, out: torch.Tensor) -> None:
+        """out = silu(norm(x) @ w[:I]^T) * (norm(x) @ w[I:]^T)"""
+        raise NotImplementedError
+
+
 class Mixer(Part):
+    # Two optional shortcuts an arrangement may take with a part that declares them:
+    # takes_pending_norm: `h` may arrive as a PendingNorm instead of normalised rows;
+    # adds_to_residual: forward accepts `residual=` (the fp32 stream) and `next_norm=` (the norm
+    #   that follows); where its last product can add into the stream and leave that norm
+    #   pending (`Norm.absorb`), it returns the PendingNorm instead of its output.
+    takes_pending_norm = False
+    adds_to_residual = False
+
     def cache_request(self) -> Optional[Any]:
         return None
 
@@ -89,6 +119,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_pending_norm = False  # as for a Mixer
+    adds_to_residual = False
+
     def forward(self, h: torch.Tensor, step: Any) -> torch.Tensor:
         raise NotImplementedError
 
@@ -96,6 +129,12 @@ class FeedForward(Part):
 class Norm(Part):
     def forward(self, x, delta=None, rows=None, update_residual=True) -> torch.Tensor:
         raise NotImplementedError
+
+    def absorb(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> Optional[PendingNorm]:
+        """x += a @ w^T (rounded as the product alone would be) with this norm of the sum left
+        pending, in one kernel; None where there is no such kernel (then the caller computes the
+        product and `forward` adds and normalises)."""
+        return None
 
 
 class Position(Part):
@@ -105,7 +144,8 @@ class Position(Part):
 
 class Arrangement:
     """Runs one layer over the residual stream `x` (fp32, updated in place) and the
-    not-yet-added output `delta` of the layer before; returns the new pending delta."""
+    not-yet-added output `delta` of the layer before (or the PendingNorm that layer left for
+    this one's `first_norm`); returns the new pending delta (or PendingNorm of `next_norm`)."""
 
     def __init__(self, spec: Any, env: BuildEnv):
         self.spec = spec
@@ -114,7 +154,11 @@ class Arrangement:
     def parts(self) -> dict:
         raise NotImplementedError
 
-    def forward(self, x, delta, step, cache):
+    def first_norm(self) -> Optional["Norm"]:
+        """The norm this layer applies to the stream first, for the layer before to leave pending."""
+        return None
+
+    def forward(self, x, delta, step, cache, next_norm=None):
         raise NotImplementedError
 
 

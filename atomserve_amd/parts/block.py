@@ -4,10 +4,12 @@
 
 The residual stream `x` is fp32 in both precisions.  A part's output is not added at
 once: it travels as the pending `delta` to the next norm, whose kernel adds it into
-`x` and normalises in one pass.
+`x` and normalises in one pass.  With few rows (decoding) both steps move into the matrix
+products around them instead: a part's last product adds into `x` and leaves the next norm
+pending (`Norm.absorb`), and the next part's first product finishes it (`PendingNorm`).
 """
 
-from atomserve_amd.parts.base import Arrangement, build, register
+from atomserve_amd.parts.base import Arrangement, PendingNorm, build, register
 
 
 class PreNormBlock(Arrangement):
@@ -21,11 +23,24 @@ class PreNormBlock(Arrangement):
     def parts(self) -> dict:
         return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "ffn_norm": self.ffn_norm, "ffn": self.ffn}
 
-    def forward(self, x, delta, step, cache):
-        h = self.mixer_norm.forward(x, delta)
-        delta = self.mixer.forward(h, step, cache)
-        h = self.ffn_norm.forward(x, delta)
-        return self.ffn.forward(h, step)
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, x, delta, step, cache, next_norm=None):
+        delta = self.apply(self.mixer_norm, self.mixer, self.ffn_norm, x, delta, step, cache)
+        return self.apply(self.ffn_norm, self.ffn, next_norm, x, delta, step)
+
+    @staticmethod
+    def apply(norm, part, next_norm, x, delta, *args):
+        """part(norm(x + delta)): the part's output still to be added, or the PendingNorm of
+        `next_norm` if the part added it itself.  `delta` may be the PendingNorm of `norm`."""
+        if isinstance(delta, PendingNorm):
+            h = delta if part.takes_pending_norm else delta.rows()
+        else:
+            h = norm.forward(x, delta)
+        if part.adds_to_residual:
+            return part.forward(h, *args, residual=x, next_norm=next_norm)
+        return part.forward(h, *args)
 
 
 register("arrangement", "prenorm", PreNormBlock)

@@ -4,10 +4,13 @@ one matrix (reference atomserve/model.py:339-360)."""
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import FeedForward, WeightDecl, register
+from atomserve_amd.parts.base import FeedForward, PendingNorm, WeightDecl, register
 
 
 class GatedMLP(FeedForward):
+    takes_pending_norm = True
+    adds_to_residual = True
+
     def __init__(self, spec, env):
         super().__init__(spec, env)
         if spec.activation != "silu":
@@ -20,12 +23,20 @@ class GatedMLP(FeedForward):
             "down.weight": WeightDecl((s.hidden_size, s.intermediate_size)),
         }
 
-    def forward(self, h, step):
+    def forward(self, h, step, residual=None, next_norm=None):
         s, env = self.spec, self.env
-        T = h.shape[0]
-        act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=h.device)
-        ops.gemm_silu_mul(h, self.gate_up_weight, act)
-        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=h.device)
+        pending = isinstance(h, PendingNorm)
+        T, device = (h.x.shape[0], h.x.device) if pending else (h.shape[0], h.device)
+        act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=device)
+        if pending:
+            h.gemm_silu_mul(self.gate_up_weight, act)
+        else:
+            ops.gemm_silu_mul(h, self.gate_up_weight, act)
+        if residual is not None and next_norm is not None:
+            link = next_norm.absorb(act, self.down_weight, residual)
+            if link is not None:
+                return link
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=device)
         ops.gemm(act, self.down_weight, y)
         return y
 

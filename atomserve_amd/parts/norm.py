@@ -6,12 +6,40 @@ pre-norm layer is fused into the same kernel: the fp32 residual stream `x` recei
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import Norm, WeightDecl, register
+from atomserve_amd.parts.base import Norm, PendingNorm, WeightDecl, register
+
+
+class PendingRMSNorm(PendingNorm):
+    """x * gain (rounded to the compute dtype) and the sums of x^2 per 16 columns: a product of
+    `scaled` times 1 / rms is the product of the normalised rows."""
+
+    def __init__(self, norm, x, scaled, ssq):
+        super().__init__(norm, x)
+        self.scaled, self.ssq = scaled, ssq
+
+    def gemm(self, w, out) -> None:
+        ops.gemm_scaled(self.scaled, self.ssq, self.norm.spec.eps, w, out)
+
+    def gemm_silu_mul(self, w, out) -> None:
+        ops.gemm_scaled(self.scaled, self.ssq, self.norm.spec.eps, w, out, gated=True)
 
 
 class RMSNorm(Norm):
     def weight_decls(self) -> dict:
         return {"weight": WeightDecl((self.spec.size,), role="vector")}
+
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        self.gain_f32 = self.weight.float()  # what the fused product reads (exact: bf16 widens)
+
+    def absorb(self, a, w, x):
+        M, N = x.shape
+        if not ops.gemm_link_supported(M, N, a.shape[1], self.env.dtype):
+            return None
+        scaled = torch.empty((M, N), dtype=self.env.dtype, device=x.device)
+        ssq = torch.empty((M, -(-N // 16)), dtype=torch.float32, device=x.device)
+        ops.gemm_link(a, w, x, self.gain_f32, scaled, ssq)
+        return PendingRMSNorm(self, x, scaled, ssq)
 
     def forward(self, x, delta=None, rows=None, update_residual=True) -> torch.Tensor:
         """x: fp32 [T, size] residual stream.  delta: pending sum in the compute dtype, or None.

@@ -263,6 +263,82 @@ def test_gemm_silu_mul_fp32(ops):
     assert torch.allclose(out, pk.silu_mul(pk.gemm(a, w)), atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1032, 4096), (16, 4096, 4096), (3, 40, 200),
+                                   (16, 24, 8), (8, 520, 12288), (13, 304, 6152), (4, 4096, 6144)])  # fmt: skip
+def test_gemm_link_bf16(ops, M, N, K):
+    """The product that adds into the fp32 stream and prepares the next norm: the stream receives
+    exactly the product kernel's bf16 output; beside it x * gain rounded to bf16 and the sums of
+    x^2 per 16 columns."""
+    assert ops.gemm_link_supported(M, N, K, BF16)
+    torch.manual_seed(12)
+    a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
+    gain = torch.randn(N, device=DEV) * 0.3 + 1
+    x0 = torch.randn(M, N, device=DEV) * 50
+    x = x0.clone()
+    scaled = torch.zeros(M, N, dtype=BF16, device=DEV)
+    strips = -(-N // 16)
+    ssq = torch.zeros(M, strips, device=DEV)
+    ops.gemm_link(a, w, x, gain, scaled, ssq)
+    y = torch.empty(M, N, dtype=BF16, device=DEV)
+    ops.gemm(a, w, y)
+    assert torch.equal(x, x0 + y.float())
+    assert torch.equal(scaled, (x * gain).to(BF16))
+    padded = torch.zeros(M, strips * 16, device=DEV)
+    padded[:, :N] = x
+    assert torch.allclose(ssq, (padded.double() ** 2).view(M, strips, 16).sum(-1).float(), rtol=1e-5)
+
+
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 6144, 4096), (9, 700, 2048),
+                                   (3, 40, 200), (16, 24, 8), (7, 264, 3072), (2, 130, 5120)])  # fmt: skip
+def test_gemm_scaled_bf16(ops, M, N, K, gated):
+    """The product that finishes a pending norm: x * gain arrives rounded to bf16, 1 / rms comes
+    from the sums of squares and multiplies the fp32 sums.  That input times the plain 1 / rms is
+    the plain norm up to its rounding; the plain product of it (and the activation) is met within
+    the product's own tolerance.  One row is a thousand times larger than the others, so a factor
+    taken from the wrong row shows."""
+    torch.manual_seed(11)
+    x = torch.randn(M, K, device=DEV) * 3
+    x[M // 2] *= 1000.0
+    gain = torch.randn(K, device=DEV) * 0.3 + 1
+    eps = 1e-5
+    w = (torch.randn((2 if gated else 1) * N, K, device=DEV) / (math.sqrt(K) if gated else 1.0)).to(BF16)
+    strips = -(-K // 16)
+    padded = torch.zeros(M, strips * 16, device=DEV)
+    padded[:, :K] = x
+    ssq = (padded**2).view(M, strips, 16).sum(-1).contiguous()
+    out = torch.empty(M, N, dtype=BF16, device=DEV)
+    # the plain norm and product, on the input as the kernel gets it: x * gain rounded to bf16
+    scaled = (x * gain).to(BF16)
+    normed, _ = pk.rmsnorm(x, gain, eps)
+    inv_rms = 1.0 / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)
+    assert close_bf16(scaled.double() * inv_rms, normed)
+    ref = ((scaled.double() @ w.double().T) * inv_rms).float()
+    ops.gemm_scaled(scaled, ssq, eps, w, out, gated=gated)
+    if not gated:
+        assert close_bf16(out, ref, scale=math.sqrt(K))
+        return
+    # each of the two products within the product's tolerance (its sums have a deviation of one
+    # here), carried through silu(g) * u: |d silu| <= 1.1 |dg|
+    g, u = ref.double().chunk(2, dim=-1)
+    err_g, err_u = g.abs() * 2.0**-7 + 2.0**-8, u.abs() * 2.0**-7 + 2.0**-8
+    silu = g / (1 + torch.exp(-g))
+    want = silu * u
+    bound = 1.1 * u.abs() * err_g + silu.abs() * err_u + 1.1 * err_g * err_u + want.abs() * 2.0**-8
+    assert bool(((out.double() - want).abs() <= bound).all())
+
+
+def test_gemm_link_refuses_what_it_cannot_do(ops):
+    assert not ops.gemm_link_supported(17, 4096, 4096, BF16)
+    assert not ops.gemm_link_supported(8, 4100, 4096, BF16)
+    assert not ops.gemm_link_supported(8, 8192, 4096, BF16)  # the next product could not keep such rows in registers
+    assert not ops.gemm_link_supported(8, 4096, 4096, F32)
+    a, w = torch.zeros(8, 64, dtype=BF16, device=DEV), torch.zeros(8192, 64, dtype=BF16, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_link(a, w, torch.zeros(8, 8192, device=DEV), torch.ones(8192, device=DEV),
+                      torch.zeros(8, 8192, dtype=BF16, device=DEV), torch.zeros(8, 512, device=DEV))
+
+
 def paged_case(dtype, H, KV, D, bs, lens, seed=0, k_scale=4.0):
     """Random pools and scattered block tables for contexts of the given lengths; the query of
     request i sits at position lens[i] - 1."""
