@@ -90,7 +90,11 @@ class StepBatch:
                 raise ValueError(f"bad row: {n} tokens at position {row.start}")
             if any(not 0 <= w < n for w in row.want):
                 raise ValueError(f"bad row: wanted places {row.want} outside its {n} tokens")
-            bad = [t for t in row.tokens if not 0 <= t < vocab_size]
+            if n > 64:  # a prompt: checked and addressed as arrays, not token by token
+                ids = np.asarray(row.tokens, dtype=np.int64)
+                bad = ids[(ids < 0) | (ids >= vocab_size)].tolist()
+            else:
+                bad = [t for t in row.tokens if not 0 <= t < vocab_size]
             if bad:
                 raise ValueError(f"token id {bad[0]} is outside the vocabulary of {vocab_size}")
             if len(row.tables) != num_paged_groups:
@@ -101,7 +105,11 @@ class StepBatch:
                 first_page, last_page = row.start // bs, (end - 1) // bs
                 if any(table[b] == RELEASED for b in range(first_page, last_page + 1)):
                     raise ValueError("block table has given back a page that this row writes")
-                if row.store:
+                if row.store and n > 64:
+                    places = np.arange(row.start, end, dtype=np.int64)
+                    pages = np.asarray(table[first_page : last_page + 1], dtype=np.int64)
+                    slots[g].extend((pages[places // bs - first_page] * bs + places % bs).tolist())
+                elif row.store:
                     slots[g].extend(table[p // bs] * bs + p % bs for p in range(row.start, end))
                 else:
                     slots[g].extend([-1] * n)

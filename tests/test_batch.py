@@ -31,6 +31,14 @@ def test_rows_are_flattened_with_slots_tables_and_tiles():
     long = pack([Row(list(range(70)), 0, [list(range(20)), list(range(20))], []), Row([1] * 9, 64, [list(range(20, 40))] * 2, [])])
     # work items of the prefill kernel, the one that sees most keys first
     assert long.long_tiles.tolist() == [[70, 9, 1, 64], [64, 6, 0, 64], [0, 64, 0, 0]]
+    # a prompt's slots are computed as arrays: the same places as token by token, from the middle of a page on
+    table = [(7 * i + 3) % 31 for i in range(30)]  # 30 different pages, in no order
+    start = BS + 3
+    prompt = pack([Row(list(range(100)), start, [table, table[::-1]], [99])])
+    for g, tb in enumerate((table, table[::-1])):
+        assert prompt.group_slots[g].tolist() == [tb[p // BS] * BS + p % BS for p in range(start, start + 100)]
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        pack([Row([1] * 80 + [-1], 0, [table, table], [])])
 
 
 def test_a_repeated_decode_step_is_updated_in_place():
