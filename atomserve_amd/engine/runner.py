@@ -60,6 +60,7 @@ class DecodeGraphs:
         r = self.runner
         return (
             r.device.type == "cuda"
+            and r.model.capturable
             and not r.manager.state_groups
             and 0 < len(rows) <= self.ROW_BUCKETS[-1]
             and all(len(row.tokens) == 1 for row in rows)

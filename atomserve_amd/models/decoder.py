@@ -24,6 +24,11 @@ class DecoderModel:
         self.embed_weight = None
         self.head_weight = None
 
+    @property
+    def capturable(self) -> bool:
+        """Whether a decode step may be captured and replayed as a graph: every part says it is."""
+        return self.final_norm.capturable and all(self.blocks[r.layer].capturable for r in self.plan.run)
+
     # ---- tensors --------------------------------------------------------------------
     def weight_decls(self) -> dict:
         p = self.plan

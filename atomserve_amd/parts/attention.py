@@ -23,6 +23,10 @@ class Attention(Mixer):
     takes_pending_norm = True
     adds_to_residual = True
 
+    @property
+    def capturable(self) -> bool:
+        return self.position is None or self.position.capturable
+
     def __init__(self, spec, env):
         super().__init__(spec, env)
         s = spec

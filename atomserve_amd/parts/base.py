@@ -60,6 +60,12 @@ class StateCacheRequest:
 class Part:
     """Common behaviour: declare tensors, receive them."""
 
+    # Whether a decode step through this part may be captured once and replayed as a graph: its
+    # work is launches on the current stream whose shapes and order depend only on the shapes of
+    # the step's tensors, with no copy to the host and no wait for the device.  A part says so
+    # itself; one that does not is run step by step.
+    capturable = False
+
     def __init__(self, spec: Any, env: "BuildEnv"):
         self.spec = spec
         self.env = env
@@ -153,6 +159,11 @@ class Arrangement:
 
     def parts(self) -> dict:
         raise NotImplementedError
+
+    @property
+    def capturable(self) -> bool:
+        """Every part of the layer is (see Part.capturable)."""
+        return all(part.capturable for part in self.parts().values())
 
     def first_norm(self) -> Optional["Norm"]:
         """The norm this layer applies to the stream first, for the layer before to leave pending."""

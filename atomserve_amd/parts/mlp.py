@@ -8,6 +8,7 @@ from atomserve_amd.parts.base import FeedForward, PendingNorm, WeightDecl, regis
 
 
 class GatedMLP(FeedForward):
+    capturable = True
     takes_pending_norm = True
     adds_to_residual = True
 

@@ -25,6 +25,8 @@ class PendingRMSNorm(PendingNorm):
 
 
 class RMSNorm(Norm):
+    capturable = True
+
     def weight_decls(self) -> dict:
         return {"weight": WeightDecl((self.spec.size,), role="vector")}
 

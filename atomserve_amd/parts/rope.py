@@ -14,6 +14,8 @@ from atomserve_amd.parts.base import Position, register
 
 
 class RotaryHalf(Position):
+    capturable = True
+
     def __init__(self, spec, env):
         super().__init__(spec, env)
         if spec.rotary_dim % 2 or spec.rotary_dim <= 0:

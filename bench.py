@@ -1,6 +1,6 @@
 """Decode and prefill throughput of random-weight Qwen3-8B layer sizes on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sizes 8b|0.6b|32b] [--batch B] [--context S]
 
 A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
 Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
@@ -22,11 +22,18 @@ if ROOT not in sys.path:
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}  # dense MFMA
 
-# Qwen3-8B layer sizes (BASELINE.json configs[2])
-SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_layers=36, num_heads=32,
-             num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
-             max_position_embeddings=40960)  # fmt: skip
-FULL_LAYERS = 36
+# Layer sizes by name; "8b" is the configuration the headline number is quoted on.
+SIZES = {
+    "8b": dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_layers=36, num_heads=32,
+               num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
+               max_position_embeddings=40960),
+    "0.6b": dict(vocab_size=151936, hidden_size=1024, intermediate_size=3072, num_layers=28, num_heads=16,
+                 num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True,
+                 max_position_embeddings=40960),
+    "32b": dict(vocab_size=151936, hidden_size=5120, intermediate_size=25600, num_layers=64, num_heads=64,
+                num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
+                max_position_embeddings=40960),
+}  # fmt: skip
 
 
 def parse_args():
@@ -36,7 +43,9 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=8)
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=2048)
-    p.add_argument("--layers", type=int, default=FULL_LAYERS)
+    p.add_argument("--sizes", choices=sorted(SIZES), default="8b", help="layer sizes of Qwen3-8B, -0.6B or -32B")
+    p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both counts are reported)")
+    p.add_argument("--max-len", type=int, default=4096, help="longest sequence the cache pool is sized for")
     p.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     p.add_argument("--points", default="1,64", help="other decode batch sizes to measure (fewer steps each)")
     p.add_argument("--no-prefill", action="store_true")
@@ -92,7 +101,8 @@ def main() -> int:
     device = "cuda:0"
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     calibration = None if args.no_calibration else calibrate(device)
-    config = Qwen3Config(**{**SIZES, "num_layers": args.layers})
+    full_layers = SIZES[args.sizes]["num_layers"]
+    config = Qwen3Config(**{**SIZES[args.sizes], "num_layers": args.layers or full_layers})
     arch = architecture_for(config.to_dict())
     model = DecoderModel(arch.build_plan(config), dtype, device)
     bind_checkpoint(model, arch, config, DictSource(random_checkpoint(arch, config, seed=0, dtype=dtype, device=device)))
@@ -100,7 +110,7 @@ def main() -> int:
 
     batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
     block = 16
-    max_len = 4096
+    max_len = max(args.max_len, args.context + args.steps + args.warmup + 16)
     num_blocks = max(batches) * max_len // block
     params = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True) if args.greedy else \
         SamplingParams(max_tokens=100000, ignore_eos=True)  # fmt: skip
@@ -168,7 +178,7 @@ def main() -> int:
     achieved = step_bytes / (ms * 1e-3)
 
     line = {
-        "metric": f"decode tok/s at batch {args.batch}, {args.context}-token contexts (Qwen3-8B sizes, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, {args.context}-token contexts (Qwen3-{args.sizes.upper()} sizes, random weights)",
         "value": round(tps, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -181,7 +191,7 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic token ids, random-init weights",
         "config": {
-            "model": "Qwen3-8B sizes", "layers": c.num_layers, "layers_full": FULL_LAYERS, "hidden": c.hidden_size,
+            "model": f"Qwen3-{args.sizes.upper()} sizes", "layers": c.num_layers, "layers_full": full_layers, "hidden": c.hidden_size,
             "heads": c.num_heads, "kv_heads": c.num_kv_heads, "head_dim": c.head_dim,
             "intermediate": c.intermediate_size, "vocab": c.vocab_size, "global_batch": args.batch,
             "seq_len": args.context, "max_context": max_len, "block_size": block, "parallelism": "single GPU",

@@ -1,7 +1,8 @@
 """Parts alone and composed: each part of a layer against its plain reference, and models
 that are not Qwen3, registered from here without a change to the package: a mixer with a
-fixed-size state of its own in some layers, a layer that runs twice, and a run that reads
-the cache another run wrote."""
+fixed-size state of its own in some layers, a feed-forward that routes each token to one of
+several experts, a position encoding that turns half of each head by slowed positions, a layer
+that runs twice, and a run that reads the cache another run wrote."""
 
 import dataclasses
 import math
@@ -321,6 +322,225 @@ def test_layers_with_a_window_have_pages_of_their_own_and_give_them_back(dtype, 
     for rc, _ in caches.values():
         m.release(rc)
     assert all(g.allocator.num_free == 24 for g in m.paged_groups)
+
+
+# ---- a toy feed-forward with routing and a toy position encoding, defined here ---------------
+
+
+@dataclasses.dataclass(frozen=True)
+class RoutedSpec:
+    kind: str
+    hidden_size: int
+    intermediate_size: int
+    num_experts: int
+
+
+@dataclasses.dataclass(frozen=True)
+class SlowedRotarySpec:
+    kind: str
+    rotary_dim: int  # the first coordinates of a head that turn; the rest stay
+    theta: float
+    slowdown: float  # positions are divided by this before the angles are formed
+
+
+def make_routed_feed_forward():
+    from atomserve_amd.parts.base import FeedForward, WeightDecl
+
+    class RoutedFeedForward(FeedForward):
+        """Each token goes to the one expert with the largest router logit (32-bit) and comes back
+        scaled by that expert's softmax weight: y = p_e * relu(h up_e^T) down_e^T."""
+
+        def weight_decls(self):
+            s = self.spec
+            return {
+                "router": WeightDecl((s.num_experts, s.hidden_size)),
+                "up": WeightDecl((s.num_experts * s.intermediate_size, s.hidden_size)),
+                "down": WeightDecl((s.num_experts * s.hidden_size, s.intermediate_size)),
+            }
+
+        def forward(self, h, step):
+            s = self.spec
+            probs = torch.softmax(h.float() @ self.router.float().T, dim=-1)
+            weight, expert = probs.max(dim=-1)
+            out = torch.zeros_like(h)
+            up = self.up.view(s.num_experts, s.intermediate_size, s.hidden_size)
+            down = self.down.view(s.num_experts, s.hidden_size, s.intermediate_size)
+            for e in range(s.num_experts):
+                rows = (expert == e).nonzero().flatten()
+                if len(rows):
+                    y = torch.relu(h[rows] @ up[e].T) @ down[e].T
+                    out[rows] = (weight[rows, None] * y.float()).to(h.dtype)
+            return out
+
+    return RoutedFeedForward
+
+
+def make_slowed_rotary():
+    from atomserve_amd.parts.base import Position
+
+    class SlowedRotary(Position):
+        """Rotation of half of each head, by angles of position / slowdown: the table the attention
+        part hands to its kernel, computed here with library calls."""
+
+        def prepare(self, step):
+            s = self.spec
+            key = ("toy_slowed", s.rotary_dim, s.theta, s.slowdown)
+            if key not in step.shared:
+                i = torch.arange(0, s.rotary_dim, 2, dtype=torch.float64, device=self.env.device)
+                angle = (step.positions.double() / s.slowdown)[:, None] / (s.theta ** (i / s.rotary_dim))[None, :]
+                step.shared[key] = torch.stack([angle.cos(), angle.sin()], dim=-1).float().contiguous()
+            return step.shared[key]
+
+    return SlowedRotary
+
+
+NUM_EXPERTS, EXPERT_WIDTH, SLOWDOWN = 3, 40, 4.0
+
+
+def register_routed_architecture():
+    """Qwen3's layers; the feed-forward of every even layer is the routed one, and the attention of
+    every odd layer turns half of each head with slowed positions."""
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+    from atomserve_amd.parts.base import register
+
+    register("feed_forward", "toy_routed", make_routed_feed_forward(), replace=True)
+    register("position", "toy_slowed", make_slowed_rotary(), replace=True)
+    qwen = architecture_for(TINY_B)
+
+    def build_plan(c):
+        plan = qwen.build_plan(c)
+        layers = []
+        for i, layer in enumerate(plan.layers):
+            if i % 2:
+                position = SlowedRotarySpec("toy_slowed", c.head_dim // 2, c.rope_theta, SLOWDOWN)
+                layer = dataclasses.replace(layer, mixer=dataclasses.replace(layer.mixer, position=position))
+            else:
+                layer = dataclasses.replace(layer, ffn=RoutedSpec("toy_routed", c.hidden_size, EXPERT_WIDTH, NUM_EXPERTS))
+            layers.append(layer)
+        return dataclasses.replace(plan, layers=tuple(layers))
+
+    def routed(c):
+        return range(0, c.num_layers, 2)
+
+    def checkpoint_map(c):
+        names = {k: v for k, v in qwen.checkpoint_map(c).items()
+                 if not any(k.startswith(f"layers.{i}.ffn.") for i in routed(c))}  # fmt: skip
+        for i in routed(c):
+            names[f"layers.{i}.ffn.router"] = [f"model.layers.{i}.moe.router.weight"]
+            names[f"layers.{i}.ffn.up"] = [f"model.layers.{i}.moe.experts.{e}.up.weight" for e in range(NUM_EXPERTS)]
+            names[f"layers.{i}.ffn.down"] = [f"model.layers.{i}.moe.experts.{e}.down.weight" for e in range(NUM_EXPERTS)]
+        return names
+
+    def checkpoint_shapes(c):
+        shapes = {k: v for k, v in qwen.checkpoint_shapes(c).items()
+                  if not any(k.startswith(f"model.layers.{i}.mlp.") for i in routed(c))}  # fmt: skip
+        for i in routed(c):
+            shapes[f"model.layers.{i}.moe.router.weight"] = ((NUM_EXPERTS, c.hidden_size), "matrix")
+            for e in range(NUM_EXPERTS):
+                shapes[f"model.layers.{i}.moe.experts.{e}.up.weight"] = ((EXPERT_WIDTH, c.hidden_size), "matrix")
+                shapes[f"model.layers.{i}.moe.experts.{e}.down.weight"] = ((c.hidden_size, EXPERT_WIDTH), "matrix")
+        return shapes
+
+    return register_architecture(
+        Architecture("ToyRoutedForCausalLM", qwen.parse_config, build_plan, checkpoint_map, checkpoint_shapes), replace=True
+    )
+
+
+def routed_weights(raw, seed):
+    w = plain_random_weights(raw, seed=seed, std=0.2, gain_std=0.2)
+    g = torch.Generator().manual_seed(seed + 100)
+    h = raw["hidden_size"]
+    for i in range(0, raw["num_hidden_layers"], 2):
+        for k in [k for k in w if k.startswith(f"model.layers.{i}.mlp.")]:
+            del w[k]
+        w[f"model.layers.{i}.moe.router.weight"] = torch.randn(NUM_EXPERTS, h, generator=g).bfloat16().float()
+        for e in range(NUM_EXPERTS):
+            w[f"model.layers.{i}.moe.experts.{e}.up.weight"] = (0.2 * torch.randn(EXPERT_WIDTH, h, generator=g)).bfloat16().float()
+            w[f"model.layers.{i}.moe.experts.{e}.down.weight"] = (0.2 * torch.randn(h, EXPERT_WIDTH, generator=g)).bfloat16().float()
+    return w
+
+
+def plain_routed_logits(raw, w, ids, slowdown=SLOWDOWN):
+    """The routed toy model, whole sequence, no cache; also the smallest lead of a chosen expert's
+    router logit over the runner-up, which says how safe the choices are from rounding."""
+    cfg = plain.normalise_config(raw)
+    wd = {k: v.double() for k, v in w.items()}
+    ids = torch.as_tensor(ids)
+    pos = torch.arange(len(ids))
+    T, H, KV, D = len(ids), cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps, theta = cfg["rms_norm_eps"], cfg["rope_theta"]
+    x = plain.embed(wd["model.embed_tokens.weight"], ids)
+    lead = math.inf
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        h = plain.rms_norm(x, wd[p + "input_layernorm.weight"], eps)
+        if i % 2:  # half of each head turns, by a quarter of the position
+            q = plain.rms_norm((h @ wd[p + "self_attn.q_proj.weight"].T).view(T, H, D), wd[p + "self_attn.q_norm.weight"], eps)
+            k = plain.rms_norm((h @ wd[p + "self_attn.k_proj.weight"].T).view(T, KV, D), wd[p + "self_attn.k_norm.weight"], eps)
+            v = (h @ wd[p + "self_attn.v_proj.weight"].T).view(T, KV, D)
+            R = D // 2
+            q = torch.cat([plain.rope(q[..., :R], pos.double() / slowdown, theta), q[..., R:]], dim=-1)
+            k = torch.cat([plain.rope(k[..., :R], pos.double() / slowdown, theta), k[..., R:]], dim=-1)
+            o = plain.causal_attention(q, k, v, pos)
+            x = x + o.reshape(T, H * D) @ wd[p + "self_attn.o_proj.weight"].T
+        else:
+            x = x + plain.attention_layer(h, wd, p, cfg, pos)
+        h = plain.rms_norm(x, wd[p + "post_attention_layernorm.weight"], eps)
+        if i % 2:
+            x = x + plain.swiglu(h, wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"], wd[p + "mlp.down_proj.weight"])
+        else:
+            scores = h @ wd[p + "moe.router.weight"].T
+            top = scores.topk(2, dim=-1).values
+            lead = min(lead, float((top[:, 0] - top[:, 1]).min()))
+            probs = torch.softmax(scores, dim=-1)
+            ys = []
+            for t in range(T):
+                e = int(probs[t].argmax())
+                y = torch.relu(h[t] @ wd[p + f"moe.experts.{e}.up.weight"].T) @ wd[p + f"moe.experts.{e}.down.weight"].T
+                ys.append(probs[t, e] * y)
+            x = x + torch.stack(ys)
+    x = plain.rms_norm(x, wd["model.norm.weight"], eps)
+    return (x @ wd["lm_head.weight"].T).float(), lead
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_feed_forward_with_routing_and_another_position_encoding(dtype, device=DEV):
+    arch = register_routed_architecture()
+    raw = {**TINY_B, "architectures": ["ToyRoutedForCausalLM"], "num_hidden_layers": 4}
+    w = routed_weights(raw, seed=42)
+    engine = build_engine(arch, raw, w, dtype, device)
+    a = torch.randint(0, 1000, (41,), generator=torch.Generator().manual_seed(6)).tolist()
+    b = torch.randint(0, 1000, (19,), generator=torch.Generator().manual_seed(7)).tolist()
+    (ref_a, lead_a), (ref_b, lead_b) = plain_routed_logits(raw, w, a), plain_routed_logits(raw, w, b)
+    assert min(lead_a, lead_b) > 0.5  # of router logits around 10: no choice of an expert hangs on rounding
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    caches = {}
+    whole = step_rows(engine, caches, [("a", a, list(range(41)))])
+    assert (whole - ref_a).abs().max() <= tol * max(1.0, ref_a.abs().max())
+    # cut anywhere and beside another request: routing is per token, angles follow the position
+    caches2, got_a, got_b = {}, [], []
+    got = step_rows(engine, caches2, [("a2", a[:9], list(range(9))), ("b", b[:2], [0, 1])])
+    got_a.append(got[:9]); got_b.append(got[9:])  # noqa: E702
+    got = step_rows(engine, caches2, [("b", b[2:18], list(range(16))), ("a2", a[9:10], [0])])
+    got_b.append(got[:16]); got_a.append(got[16:])  # noqa: E702
+    got = step_rows(engine, caches2, [("a2", a[10:], list(range(31))), ("b", b[18:], [0])])
+    got_a.append(got[:31]); got_b.append(got[31:])  # noqa: E702
+    assert (torch.cat(got_a) - ref_a).abs().max() <= tol * max(1.0, ref_a.abs().max())
+    assert (torch.cat(got_b) - ref_b).abs().max() <= tol * max(1.0, ref_b.abs().max())
+    # through the scheduler: decode steps of a model with a part that cannot be captured run eagerly
+    assert not engine.runner.model.capturable
+    if dtype == torch.float32:
+        from atomserve_amd.engine.sequence import SamplingParams
+
+        outs = engine.generate([a[:7], b[:12]], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))
+        for prompt, out in zip((a[:7], b[:12]), outs):
+            seq = list(prompt)
+            for t in out:
+                assert t == int(plain_routed_logits(raw, w, seq)[0][-1].argmax())
+                seq.append(t)
+    # the test would not pass with the wrong angles: without the slowdown the logits move by 2.4,
+    # ten times what the comparison above allows in bfloat16
+    assert (plain_routed_logits(raw, w, a, slowdown=1.0)[0] - ref_a).abs().max() > 8 * 3e-2 * ref_a.abs().max()
 
 
 # ---- each part alone ------------------------------------------------------------------------
