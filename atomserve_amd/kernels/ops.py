@@ -16,21 +16,29 @@ _DT = {F32: 0, BF16: 1}
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The raw handle of torch's current stream on the current device (an eager step makes some
+    hundred launches, so this asks the binding directly instead of building a Stream object)."""
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 def _check(t, name, dtype=None, shape=None):
+    """Runs before every launch, several times: written for the case that all is well."""
     if not isinstance(t, torch.Tensor) or not t.is_cuda:
         raise KernelError(f"{name} must be a tensor on the GPU")
     if not t.is_contiguous():
         raise KernelError(f"{name} must be contiguous")
-    if dtype is not None:
-        allowed = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
-        if t.dtype not in allowed:
-            raise KernelError(f"{name} has dtype {t.dtype}, expected {allowed}")
+    if dtype is not None and t.dtype is not dtype and (isinstance(dtype, torch.dtype) or t.dtype not in dtype):
+        raise KernelError(f"{name} has dtype {t.dtype}, expected {dtype}")
     if shape is not None:
-        if t.dim() != len(shape) or any(s is not None and int(d) != int(s) for d, s in zip(t.shape, shape)):
-            raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+        have = t.shape
+        good = len(have) == len(shape)
+        if good:
+            for d, s in zip(have, shape):
+                if s is not None and d != s:
+                    good = False
+                    break
+        if not good:
+            raise KernelError(f"{name} has shape {tuple(have)}, expected {tuple(shape)}")
 
 
 def _ptr(t) -> int:
