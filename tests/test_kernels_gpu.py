@@ -159,6 +159,13 @@ def test_qk_norm_rope_store_many_tokens_bf16(ops, D, bs, gain, rope):
     q2 = torch.empty_like(q)
     ops.qk_norm_rope_store(qkv, qw, kw, cs, None, q2, None, None, H, KV, 1e-6, store_kv=False)
     assert torch.equal(q2, q)
+    # a prompt's own layout: slots that follow one another from the middle of a page on
+    run = list(range(5, 5 + T))
+    k_run, v_run = torch.zeros_like(k_pages), torch.zeros_like(v_pages)
+    ops.qk_norm_rope_store(qkv, qw, kw, cs, i32(run), q2, k_run, v_run, H, KV, 1e-6)
+    ref_k.zero_(), ref_v.zero_()
+    pk.store_pages(ref_k, ref_v, rk, rv, i32(run))
+    assert close_bf16(k_run, ref_k) and torch.equal(v_run.float(), ref_v)
 
 
 def test_qk_norm_rope_store_variants(ops):
