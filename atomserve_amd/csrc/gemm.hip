@@ -257,7 +257,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(const b
     const int l = e & 63, tile = e >> 6, s = tile / MT, mt = tile % MT;
     const int m = mt * 16 + (l & 15), n = n0 + s * 16 + 4 * (l >> 4);
     if constexpr (LINK) {
-      static_assert(!LINK || (S == 1 && MT == 1), "one strip, one wave of lanes");
+      static_assert(!LINK || S == 1, "one strip a workgroup: its index names the sums of squares");
       link_epilogue(link, reinterpret_cast<float*>(out), sum, m, n, M, N, blockIdx.x, gridDim.x);
     } else {
       if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
@@ -296,12 +296,13 @@ static int launch_skinny(const void* a, const void* w, void* out, int out_dtype,
 // the same outputs); the wave whose turn it is keeps the gate sums until the up sums arrive.
 constexpr int PIPE_WAVES = 8;
 constexpr int PIPE_MAX_NST = 12;
+constexpr int PIPE_MAX_NST_TWO = 8;  // with two row tiles
 
 template <typename OutT> __device__ __forceinline__ float rounded(float v);
 template <> __device__ __forceinline__ float rounded<float>(float v) { return v; }
 template <> __device__ __forceinline__ float rounded<bf16>(float v) { return (float)(bf16)v; }
 
-template <int NST, bool MASKED, bool GATED, typename OutT, bool SCALED = false, bool LINK = false>
+template <int NST, bool MASKED, bool GATED, typename OutT, bool SCALED = false, bool LINK = false, int MT = 1>
 __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(const bf16* __restrict__ a,
                                                                                const bf16* __restrict__ w,
                                                                                OutT* __restrict__ out, int M, int N,
@@ -310,8 +311,8 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
   static_assert(NST % 2 == 0, "a wave's slice is handled in two halves");
   static_assert(!LINK || (!GATED && !SCALED && sizeof(OutT) == 4), "the stream is fp32 and takes a plain product");
   constexpr int H = NST / 2;
-  __shared__ floatx4 red[2][PIPE_WAVES * 64];
-  __shared__ float inv_rms[16];
+  __shared__ floatx4 red[2][MT][PIPE_WAVES * 64];
+  __shared__ float inv_rms[16 * MT];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
   const int kbase = wave * NST * 64 + lg * 16;  // this lane's first k; step u adds 64 u
@@ -327,68 +328,79 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
     BUF[u][0] = PIPE_VALID((OFF) + u, 0) ? *reinterpret_cast<const bf16x8*>(ROW + ((OFF) + u) * 64) : zero;   \
     BUF[u][1] = PIPE_VALID((OFF) + u, 1) ? *reinterpret_cast<const bf16x8*>(ROW + ((OFF) + u) * 64 + 8) : zero; \
   }
-#define PIPE_MATH(BUF, OFF)                                                                   \
-  _Pragma("unroll") for (int u = 0; u < H; ++u) {                                             \
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][0], av[(OFF) + u][0], acc, 0, 0, 0); \
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][1], av[(OFF) + u][1], acc, 0, 0, 0); \
+#define PIPE_MATH(BUF, OFF)                                                                                   \
+  _Pragma("unroll") for (int u = 0; u < H; ++u) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {             \
+    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][0], av[mt][(OFF) + u][0], acc[mt], 0, 0, 0);       \
+    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][1], av[mt][(OFF) + u][1], acc[mt], 0, 0, 0);       \
   }
 #define PIPE_ROWS(STRIP, UP) (w + ((size_t)min((STRIP) * 16 + lr, N - 1) + ((UP) ? (size_t)N : 0)) * K + kbase)
   bf16x8 w0[H][2], w1[H][2];
   const bf16* wrow = PIPE_ROWS(strip, false);
   PIPE_LOAD(w0, wrow, 0)
   PIPE_LOAD(w1, wrow, H)
-  bf16x8 av[NST][2];
-  {
-    const bf16* arow = a + (size_t)min(lr, M - 1) * K + kbase;
+  bf16x8 av[MT][NST][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const bf16* arow = a + (size_t)min(mt * 16 + lr, M - 1) * K + kbase;
 #pragma unroll
     for (int u = 0; u < NST; ++u) {
-      av[u][0] = PIPE_VALID(u, 0) ? *reinterpret_cast<const bf16x8*>(arow + u * 64) : zero;
-      av[u][1] = PIPE_VALID(u, 1) ? *reinterpret_cast<const bf16x8*>(arow + u * 64 + 8) : zero;
+      av[mt][u][0] = PIPE_VALID(u, 0) ? *reinterpret_cast<const bf16x8*>(arow + u * 64) : zero;
+      av[mt][u][1] = PIPE_VALID(u, 1) ? *reinterpret_cast<const bf16x8*>(arow + u * 64 + 8) : zero;
     }
   }
   if constexpr (SCALED) {
-    // 1 / rms of the 16 rows, 32 threads a row; published by the first strip's barrier
-    const int row = threadIdx.x >> 5, j0 = threadIdx.x & 31;
-    float ss = 0.f;
-    if (row < M)
-      for (int j = j0; j < link.strips_in; j += 32) ss += link.ssq_in[(size_t)row * link.strips_in + j];
+    // 1 / rms of the rows, 32 threads a row and 16 rows at a time; published by the first strip's barrier
+    const int j0 = threadIdx.x & 31;
 #pragma unroll
-    for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off, 64);
-    if (j0 == 0) inv_rms[row] = row < M ? 1.0f / sqrtf(ss / (float)K + link.eps) : 0.f;
+    for (int mt = 0; mt < MT; ++mt) {
+      const int row = mt * 16 + (threadIdx.x >> 5);
+      float ss = 0.f;
+      if (row < M)
+        for (int j = j0; j < link.strips_in; j += 32) ss += link.ssq_in[(size_t)row * link.strips_in + j];
+#pragma unroll
+      for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off, 64);
+      if (j0 == 0) inv_rms[row] = row < M ? 1.0f / sqrtf(ss / (float)K + link.eps) : 0.f;
+    }
   }
   int buf = 0, turn = 0;
-  floatx4 gate = {0.f, 0.f, 0.f, 0.f};
+  floatx4 gate[MT];
   for (;;) {
     const bool next_up = GATED && !up;
     const int next = next_up ? strip : strip + gridDim.x;
     const bool more = next < nstrips;
     const bf16* nrow = PIPE_ROWS(next, next_up);
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    floatx4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
     PIPE_MATH(w0, 0)
     if (more) { PIPE_LOAD(w0, nrow, 0) }
     PIPE_MATH(w1, H)
     if (more) { PIPE_LOAD(w1, nrow, H) }
-    red[buf][wave * 64 + lane] = acc;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[buf][mt][wave * 64 + lane] = acc[mt];
     __syncthreads();
     if (wave == turn) {  // sums in the order of the waves, whichever wave adds them
-      floatx4 sum = red[buf][lane];
 #pragma unroll
-      for (int x = 1; x < PIPE_WAVES; ++x) sum += red[buf][x * 64 + lane];
-      if constexpr (SCALED) sum *= inv_rms[lr];
-      const int m = lr, n = strip * 16 + 4 * lg;
-      if constexpr (LINK) {
-        link_epilogue(link, reinterpret_cast<float*>(out), sum, m, n, M, N, strip, nstrips);
-      } else if (GATED && !up) {
-        gate = sum;
-      } else {
-        if (GATED) {
+      for (int mt = 0; mt < MT; ++mt) {
+        floatx4 sum = red[buf][mt][lane];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float g = rounded<OutT>(gate[r]);
-            sum[r] = g / (1.0f + expf(-g)) * rounded<OutT>(sum[r]);
+        for (int x = 1; x < PIPE_WAVES; ++x) sum += red[buf][mt][x * 64 + lane];
+        const int m = mt * 16 + lr, n = strip * 16 + 4 * lg;
+        if constexpr (SCALED) sum *= inv_rms[m];
+        if constexpr (LINK) {
+          link_epilogue(link, reinterpret_cast<float*>(out), sum, m, n, M, N, strip, nstrips);
+        } else if (GATED && !up) {
+          gate[mt] = sum;
+        } else {
+          if (GATED) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float g = rounded<OutT>(gate[mt][r]);
+              sum[r] = g / (1.0f + expf(-g)) * rounded<OutT>(sum[r]);
+            }
           }
+          if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
         }
-        if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
       }
     }
     if (!more) break;
@@ -405,36 +417,53 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
 #undef PIPE_MATH
 }
 
-template <int NST, bool GATED, typename OutT, bool SCALED, bool LINK>
+template <int NST, bool GATED, typename OutT, bool SCALED, bool LINK, int MT>
 static int launch_pipe(const void* a, const void* w, void* out, int M, int N, int K, const NormLink& link,
                        hipStream_t stream) {
   const int nstrips = (N + 15) / 16;
   const int blocks = min(nstrips, compute_units());
   if (K == 64 * PIPE_WAVES * NST)
-    gemm_bf16_skinny_pipe_kernel<NST, false, GATED, OutT, SCALED, LINK><<<blocks, PIPE_WAVES * 64, 0, stream>>>(
+    gemm_bf16_skinny_pipe_kernel<NST, false, GATED, OutT, SCALED, LINK, MT><<<blocks, PIPE_WAVES * 64, 0, stream>>>(
         (const bf16*)a, (const bf16*)w, (OutT*)out, M, N, K, nstrips, link);
   else
-    gemm_bf16_skinny_pipe_kernel<NST, true, GATED, OutT, SCALED, LINK><<<blocks, PIPE_WAVES * 64, 0, stream>>>(
+    gemm_bf16_skinny_pipe_kernel<NST, true, GATED, OutT, SCALED, LINK, MT><<<blocks, PIPE_WAVES * 64, 0, stream>>>(
         (const bf16*)a, (const bf16*)w, (OutT*)out, M, N, K, nstrips, link);
   return launch_status();
+}
+
+// Whether the persistent kernel takes a product of these sizes: the activations of a wave's
+// K-slice stay in its registers, 8 per row tile and 64 columns, so 17 to 32 rows (two row tiles)
+// leave room for K up to 64 * PIPE_WAVES * PIPE_MAX_NST_TWO only.  (Whether two row tiles pay is
+// the caller's question: every workgroup reads all rows of the activations, which at 32 rows
+// and K = 4096 is more than its share of the weights.)
+static bool pipe_fits(int M, int K) {
+  return (M <= 16 && K <= 64 * PIPE_WAVES * PIPE_MAX_NST) || (M <= 32 && K <= 64 * PIPE_WAVES * PIPE_MAX_NST_TWO);
 }
 
 template <bool GATED, typename OutT, bool SCALED = false, bool LINK = false>
 static int dispatch_pipe(const void* a, const void* w, void* out, int M, int N, int K, hipStream_t stream,
                          const NormLink& link = NormLink{}) {
-  switch (2 * ((K + 128 * PIPE_WAVES - 1) / (128 * PIPE_WAVES))) {
-    case 2: return launch_pipe<2, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
-    case 4: return launch_pipe<4, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
-    case 6: return launch_pipe<6, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
-    case 8: return launch_pipe<8, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
-    case 10: return launch_pipe<10, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
-    case 12: return launch_pipe<12, GATED, OutT, SCALED, LINK>(a, w, out, M, N, K, link, stream);
+  if (!pipe_fits(M, K)) return AS_BAD_SHAPE;
+  const int nst = 2 * ((K + 128 * PIPE_WAVES - 1) / (128 * PIPE_WAVES));
+  if (M > 16) {
+    switch (nst) {
+      case 2: return launch_pipe<2, GATED, OutT, SCALED, LINK, 2>(a, w, out, M, N, K, link, stream);
+      case 4: return launch_pipe<4, GATED, OutT, SCALED, LINK, 2>(a, w, out, M, N, K, link, stream);
+      case 6: return launch_pipe<6, GATED, OutT, SCALED, LINK, 2>(a, w, out, M, N, K, link, stream);
+      case 8: return launch_pipe<8, GATED, OutT, SCALED, LINK, 2>(a, w, out, M, N, K, link, stream);
+    }
+    return AS_BAD_SHAPE;
+  }
+  switch (nst) {
+    case 2: return launch_pipe<2, GATED, OutT, SCALED, LINK, 1>(a, w, out, M, N, K, link, stream);
+    case 4: return launch_pipe<4, GATED, OutT, SCALED, LINK, 1>(a, w, out, M, N, K, link, stream);
+    case 6: return launch_pipe<6, GATED, OutT, SCALED, LINK, 1>(a, w, out, M, N, K, link, stream);
+    case 8: return launch_pipe<8, GATED, OutT, SCALED, LINK, 1>(a, w, out, M, N, K, link, stream);
+    case 10: return launch_pipe<10, GATED, OutT, SCALED, LINK, 1>(a, w, out, M, N, K, link, stream);
+    case 12: return launch_pipe<12, GATED, OutT, SCALED, LINK, 1>(a, w, out, M, N, K, link, stream);
   }
   return AS_BAD_SHAPE;
 }
-
-// Whether the persistent kernel takes a product of these sizes.
-static bool pipe_fits(int M, int K) { return M <= 16 && K <= 64 * PIPE_WAVES * PIPE_MAX_NST; }
 
 // out[M, N] = silu(a @ w[:N]^T) * (a @ w[N:]^T) for w[2N, K] in bf16, both products rounded
 // to bf16 before the activation.  Only sizes of the persistent kernel; AS_BAD_SHAPE
@@ -447,21 +476,24 @@ extern "C" int as_gemm_bf16_gated(const void* a, const void* w, void* out, int M
 }
 
 // The producer of a NormLink: x[M, N] (fp32) += bf16(a @ w^T); scaled[M, N] = bf16(x * gain);
-// ssq[M, ceil(N / 16)] = sums of x^2 per 16 columns.  M <= 16, K % 8 == 0, N % 4 == 0; a K beyond
+// ssq[M, ceil(N / 16)] = sums of x^2 per 16 columns.  M <= 32, K % 8 == 0, N % 4 == 0; a K beyond
 // the persistent kernel goes through the streaming one.
 extern "C" int as_gemm_bf16_link(const void* a, const void* w, float* x, const float* gain, void* scaled,
                                  float* ssq, int M, int N, int K, hipStream_t stream) {
   if (M <= 0) return AS_OK;
-  if (M > 16 || N <= 0 || K <= 0 || (K & 7) || (N & 3) || !gain || !scaled || !ssq) return AS_BAD_SHAPE;
+  if (M > 32 || N <= 0 || K <= 0 || (K & 7) || (N & 3) || !gain || !scaled || !ssq) return AS_BAD_SHAPE;
   const NormLink link{nullptr, 0, 0.f, gain, (bf16*)scaled, ssq};
   if (pipe_fits(M, K)) return dispatch_pipe<false, float, false, true>(a, w, x, M, N, K, stream, link);
   const int blocks = (N + 15) / 16;
-  if (blocks < 512)
-    gemm_bf16_skinny_kernel<1, 1, 16, float, true><<<blocks, 16 * 64, sizeof(floatx4) * 16 * 64, stream>>>(
-        (const bf16*)a, (const bf16*)w, x, M, N, K, link);
-  else
-    gemm_bf16_skinny_kernel<1, 1, 8, float, true><<<blocks, 8 * 64, sizeof(floatx4) * 8 * 64, stream>>>(
-        (const bf16*)a, (const bf16*)w, x, M, N, K, link);
+#define LINK_STREAM(MTV, WAVES)                                                                                 \
+  gemm_bf16_skinny_kernel<1, MTV, WAVES, float, true><<<blocks, WAVES * 64, sizeof(floatx4) * WAVES * MTV * 64, stream>>>( \
+      (const bf16*)a, (const bf16*)w, x, M, N, K, link)
+  if (M <= 16) {
+    if (blocks < 512) LINK_STREAM(1, 16); else LINK_STREAM(1, 8);
+  } else {
+    if (blocks < 512) LINK_STREAM(2, 16); else LINK_STREAM(2, 8);
+  }
+#undef LINK_STREAM
   return launch_status();
 }
 

@@ -228,6 +228,25 @@ def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, m
 
 
 SKINNY_MAX_ROWS = 16  # up to here the bf16 product streams the weights through our own kernel
+# 17 to 32 rows: the persistent kernel keeps two row tiles in registers up to this K ...
+SKINNY_TWO_MAX_ROWS, SKINNY_TWO_MAX_K = 32, 4096
+# ... and pays while the activations, which EVERY workgroup reads whole, stay a fraction of the
+# weights' bytes: at 32 rows of 4096 over 256 workgroups (67 MB) the library's product is faster,
+# with rows of 1024 (17 MB) this one is, by the two kernels it saves beside.
+SKINNY_TWO_MAX_ACT_BYTES = 36 << 20
+WORKGROUPS = 256  # persistent kernels run one workgroup per compute unit
+
+
+def _few_rows(rows: int, k: int, n: int, max_k=None) -> bool:
+    """Whether a product of `rows` rows of width `k` with `n` output columns goes through the
+    few-rows kernels of this package."""
+    if rows <= 0 or k % 8:
+        return False
+    if rows <= SKINNY_MAX_ROWS:
+        return max_k is None or k <= max_k
+    strips = min(-(-n // 16), WORKGROUPS)
+    return (rows <= SKINNY_TWO_MAX_ROWS and k <= SKINNY_TWO_MAX_K
+            and strips * rows * k * 2 <= SKINNY_TWO_MAX_ACT_BYTES)  # fmt: skip
 
 
 def gemm(a, w, out) -> None:
@@ -246,7 +265,7 @@ def gemm(a, w, out) -> None:
         return
     if out.dtype not in (BF16, F32):
         raise KernelError(f"gemm: unsupported output dtype {out.dtype}")
-    if M <= SKINNY_MAX_ROWS and K % 8 == 0:
+    if _few_rows(M, K, N):
         call("as_gemm_bf16_skinny", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, 0, _stream())
     elif out.dtype == BF16:
         torch.mm(a, w.t(), out=out)
@@ -268,7 +287,7 @@ def gemm_silu_mul(a, w, out) -> None:
     _check(w, "w", a.dtype, (2 * inter, K))
     if M == 0:
         return
-    if a.dtype == BF16 and M <= SKINNY_MAX_ROWS and K % 8 == 0 and K <= GATED_MAX_K:
+    if a.dtype == BF16 and _few_rows(M, K, inter, GATED_MAX_K):
         call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), M, inter, K, _stream())
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
@@ -279,8 +298,16 @@ def gemm_silu_mul(a, w, out) -> None:
 def gemm_link_supported(rows: int, n_out: int, k: int, dtype) -> bool:
     """Whether `gemm_link` and, for its result, `gemm_scaled` exist: bf16, few rows, widths the
     kernels take (n_out is the width of the stream, which is the next product's input)."""
-    return (dtype == BF16 and 0 < rows <= SKINNY_MAX_ROWS and k % 8 == 0 and n_out % 8 == 0
-            and n_out <= GATED_MAX_K)  # fmt: skip
+    if dtype != BF16 or rows <= 0 or k % 8 or n_out % 8 or n_out > GATED_MAX_K:
+        return False
+    if rows <= SKINNY_MAX_ROWS:
+        return True
+    # two row tiles: the producer reads its activations once per strip of 16 outputs (whole rows
+    # for every workgroup of the persistent kernel, and for every strip beyond its K), the consumer
+    # keeps rows of n_out in registers in each of its workgroups
+    producer_strips = -(-n_out // 16) if k > SKINNY_TWO_MAX_K else min(-(-n_out // 16), WORKGROUPS)
+    return (rows <= SKINNY_TWO_MAX_ROWS and producer_strips * rows * k * 2 <= SKINNY_TWO_MAX_ACT_BYTES
+            and _few_rows(rows, n_out, 16 * WORKGROUPS))  # fmt: skip
 
 
 def gemm_link(a, w, x, gain, scaled, ssq) -> None:

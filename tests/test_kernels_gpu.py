@@ -229,7 +229,8 @@ def test_gemm_fp32_rows_do_not_depend_on_the_batch(ops):
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (64, 4096, 1024), (300, 257, 192), (5, 2000, 4096),
                                    (16, 4096, 4096), (12, 8200, 4096), (9, 16000, 2048), (3, 40, 200), (16, 24, 8),
                                    (4, 1040, 5120), (7, 520, 6144), (2, 100, 2560), (11, 4100, 3072), (8, 512, 12288),
-                                   (13, 300, 6152), (17, 300, 4096)])  # fmt: skip
+                                   (13, 300, 6152), (17, 300, 4096), (32, 6144, 1024), (25, 1000, 1000),
+                                   (31, 520, 3072), (20, 64, 4096), (32, 300, 24), (32, 6144, 4096)])  # fmt: skip
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(8)
     a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
@@ -244,7 +245,8 @@ def test_gemm_bf16(ops, M, N, K):
 
 @pytest.mark.parametrize("M,I,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 12288, 4096), (9, 700, 2048),
                                    (3, 40, 200), (16, 24, 8), (4, 520, 5120), (7, 264, 6144), (8, 128, 12288),
-                                   (40, 300, 512)])  # fmt: skip
+                                   (40, 300, 512), (32, 1030, 2048), (17, 264, 2048), (29, 128, 4096),
+                                   (24, 72, 200)])  # fmt: skip
 def test_gemm_silu_mul_bf16(ops, M, I, K):
     """Gate and up products with the activation in one kernel (few rows, an input that fits)
     or as product then activation: the same numbers as the two kernels give, which are the plain
@@ -271,7 +273,8 @@ def test_gemm_silu_mul_fp32(ops):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1032, 4096), (16, 4096, 4096), (3, 40, 200),
-                                   (16, 24, 8), (8, 520, 12288), (13, 304, 6152), (4, 4096, 6144)])  # fmt: skip
+                                   (16, 24, 8), (8, 520, 12288), (13, 304, 6152), (4, 4096, 6144), (32, 1024, 4096),
+                                   (17, 1032, 12288), (27, 520, 200), (32, 2048, 4104), (20, 40, 2048)])  # fmt: skip
 def test_gemm_link_bf16(ops, M, N, K):
     """The product that adds into the fp32 stream and prepares the next norm: the stream receives
     exactly the product kernel's bf16 output; beside it x * gain rounded to bf16 and the sums of
@@ -286,9 +289,12 @@ def test_gemm_link_bf16(ops, M, N, K):
     strips = -(-N // 16)
     ssq = torch.zeros(M, strips, device=DEV)
     ops.gemm_link(a, w, x, gain, scaled, ssq)
-    y = torch.empty(M, N, dtype=BF16, device=DEV)
-    ops.gemm(a, w, y)
-    assert torch.equal(x, x0 + y.float())
+    if M <= 16 or (K <= ops.SKINNY_TWO_MAX_K and ops._few_rows(M, K, N)):  # the plain product sums in the same order
+        y = torch.empty(M, N, dtype=BF16, device=DEV)
+        ops.gemm(a, w, y)
+        assert torch.equal(x, x0 + y.float())
+    else:  # what the stream received is the product rounded to bf16 (the fp32 sum's own rounding is far below)
+        assert close_bf16(x - x0, pk.gemm(a, w), scale=math.sqrt(K))
     assert torch.equal(scaled, (x * gain).to(BF16))
     padded = torch.zeros(M, strips * 16, device=DEV)
     padded[:, :N] = x
@@ -297,7 +303,8 @@ def test_gemm_link_bf16(ops, M, N, K):
 
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 6144, 4096), (9, 700, 2048),
-                                   (3, 40, 200), (16, 24, 8), (7, 264, 3072), (2, 130, 5120)])  # fmt: skip
+                                   (3, 40, 200), (16, 24, 8), (7, 264, 3072), (2, 130, 5120), (32, 6144, 1024),
+                                   (17, 1030, 2048), (26, 40, 200), (31, 264, 2048)])  # fmt: skip
 def test_gemm_scaled_bf16(ops, M, N, K, gated):
     """The product that finishes a pending norm: x * gain arrives rounded to bf16, 1 / rms comes
     from the sums of squares and multiplies the fp32 sums.  That input times the plain 1 / rms is
@@ -336,7 +343,9 @@ def test_gemm_scaled_bf16(ops, M, N, K, gated):
 
 
 def test_gemm_link_refuses_what_it_cannot_do(ops):
-    assert not ops.gemm_link_supported(17, 4096, 4096, BF16)
+    assert not ops.gemm_link_supported(33, 1024, 1024, BF16)
+    assert not ops.gemm_link_supported(32, 4096, 4096, BF16)  # two row tiles of such rows in 256 workgroups: more bytes than the weights
+    assert ops.gemm_link_supported(32, 1024, 3072, BF16)
     assert not ops.gemm_link_supported(8, 4100, 4096, BF16)
     assert not ops.gemm_link_supported(8, 8192, 4096, BF16)  # the next product could not keep such rows in registers
     assert not ops.gemm_link_supported(8, 4096, 4096, F32)

@@ -97,12 +97,13 @@ def test_decoding_across_the_context_bound_of_a_captured_graph(dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("num_requests", [3, 13, 40])
+@pytest.mark.parametrize("num_requests", [3, 13, 21, 40])
 def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
     """Decode steps replayed as captured graphs against the same steps launched kernel by kernel:
     the same logits at every step, over several replays with eager work (a new request's prompt)
-    and synchronisations between them, for row counts in the small buckets and the large ones
-    (whose matrix products are the library's)."""
+    and synchronisations between them, for row counts in the small buckets (one and two row tiles
+    of this package's products) and the large ones (whose matrix products are the library's).  The
+    last step's logits are also the plain model's."""
     from atomserve_amd.cache.manager import CacheManager
     from atomserve_amd.engine.batch import Row
     from atomserve_amd.engine.runner import ModelRunner
@@ -143,6 +144,10 @@ def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
     for a, b in zip(seen[True], seen[False]):
         assert a.shape == b.shape and torch.isfinite(a).all()
         check(float((a - b).abs().max()), float(b.abs().max()), dtype)
+    for i in (0, num_requests // 2, num_requests - 1):
+        ref = plain.logits(raw, weights, prompts[i] + later[i][:8])[-1].float()
+        for out in seen.values():
+            check(float((out[-1][i] - ref).abs().max()), float(ref.abs().max()), dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
