@@ -1,6 +1,7 @@
 """Decode and prefill throughput of random-weight Qwen3-8B layer sizes on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sizes 8b|0.6b|32b] [--batch B] [--context S]
+    python bench.py --workload mixed --sizes 0.6b      (a continuous batch through the scheduler)
 
 A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
 Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
@@ -51,12 +52,84 @@ def parse_args():
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--no-calibration", action="store_true", help="skip the library copy and matmul probes")
     p.add_argument("--greedy", action="store_true", help="greedy instead of the default sampling settings")
+    p.add_argument("--workload", choices=["decode", "mixed"], default="decode",
+                   help="decode: the timed decode steps above; mixed: 32 requests with prompts of 64 to 2,048 tokens "
+                        "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
+                        "scheduler from submission to the last token")  # fmt: skip
     return p.parse_args()
 
 
 def prompt(b: int, n: int, vocab: int) -> list:
     """Distinct synthetic prompts (reference bench/engine.py:90-92)."""
     return [(1000 + 37 * b + i) % (vocab - 1000) for i in range(n)]
+
+
+def mixed_workload(args, model, config, full_layers: int) -> dict:
+    """A continuous batch as a server sees it: everything is submitted at once, prompts are cut
+    into portions under the token budget beside the running requests' decode steps, prefixes are
+    reused.  One untimed run first (graphs are captured, libraries pick their kernels), then the
+    median of three runs with other prompts of the same lengths' distribution."""
+    import random
+
+    import torch
+
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+
+    requests, longest, decoded, budget, block = 32, 2048, 128, 512, 16
+    max_len = longest + decoded + block
+    engine = create_engine(model, EngineConfig(block_size=block, num_blocks=requests * max_len // block,
+                                               max_num_seqs=requests, max_num_batched_tokens=budget,
+                                               max_model_len=max_len, enable_prefix_caching=True), seed=0)  # fmt: skip
+    params = SamplingParams(temperature=0.0, max_tokens=decoded, ignore_eos=True) if args.greedy else \
+        SamplingParams(max_tokens=decoded, ignore_eos=True)  # fmt: skip
+    rng = random.Random(0)
+
+    def run():
+        prefix = [rng.randrange(1000, config.vocab_size - 1000) for _ in range(32)]
+        prompts = []
+        for i in range(requests):
+            body = [rng.randrange(1000, config.vocab_size - 1000) for _ in range(rng.randint(64, longest))]
+            prompts.append(prefix + body[32:] if i % 2 == 0 else body)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for p in prompts:
+            engine.submit(p, params)
+        steps = 0
+        while engine.step():
+            steps += 1
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, sum(map(len, prompts)), steps
+
+    run()
+    dt, prompt_tokens, steps = sorted(run() for _ in range(3))[1]
+    c = config
+    return {
+        "metric": f"generated tok/s of a mixed continuous batch (Qwen3-{args.sizes.upper()} sizes, random weights)",
+        "value": round(requests * decoded / dt, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": 1,
+        "ms_per_step": round(dt / steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic token ids, random-init weights",
+        "config": {
+            "model": f"Qwen3-{args.sizes.upper()} sizes", "layers": c.num_layers, "layers_full": full_layers,
+            "hidden": c.hidden_size, "heads": c.num_heads, "kv_heads": c.num_kv_heads, "head_dim": c.head_dim,
+            "intermediate": c.intermediate_size, "vocab": c.vocab_size, "global_batch": requests,
+            "seq_len": longest, "decoded_each": decoded, "chunk_budget": budget, "block_size": block,
+            "shared_prefix": 32, "parallelism": "single GPU",
+            "sampling": "greedy" if args.greedy else "temperature 0.6 top-k 20 top-p 0.95",
+        },
+        "run_ms": round(dt * 1e3, 1),
+        "prompt_tokens": prompt_tokens,
+        "all_tokens_per_s": round((prompt_tokens + requests * decoded) / dt, 1),
+    }
 
 
 def calibrate(device) -> dict:
@@ -107,6 +180,9 @@ def main() -> int:
     model = DecoderModel(arch.build_plan(config), dtype, device)
     bind_checkpoint(model, arch, config, DictSource(random_checkpoint(arch, config, seed=0, dtype=dtype, device=device)))
     torch.cuda.synchronize()
+    if args.workload == "mixed":
+        print(json.dumps(mixed_workload(args, model, config, full_layers)))
+        return 0
 
     batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
     block = 16
