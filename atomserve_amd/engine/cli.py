@@ -34,7 +34,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--max-num-seqs", type=int, default=32, help="most requests running at once")
     p.add_argument("--max-batched-tokens", type=int, default=512,
                    help="token budget of one forward pass; smaller bounds the stall a long prompt causes "
-                        "running streams, larger prefills a little faster")  # fmt: skip
+                        "running streams, larger prefills faster (on an MI355X 2048 gives a mixed batch of "
+                        "Qwen3-8B size a fifth more throughput than 512, for steps of 28 ms instead of 12)")  # fmt: skip
     p.add_argument("--no-prefix-caching", action="store_true", help="always recompute shared prompt prefixes")
     p.add_argument("--max-model-len", type=int, default=None, help="longest sequence accepted (default: what model and pool allow)")
     p.add_argument("--random-weights", type=int, default=None, metavar="SEED",
