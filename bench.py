@@ -56,6 +56,7 @@ def parse_args():
                    help="decode: the timed decode steps above; mixed: 32 requests with prompts of 64 to 2,048 tokens "
                         "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
                         "scheduler from submission to the last token")  # fmt: skip
+    p.add_argument("--chunk-budget", type=int, default=512, help="token budget of a step in the mixed workload")
     return p.parse_args()
 
 
@@ -77,7 +78,7 @@ def mixed_workload(args, model, config, full_layers: int) -> dict:
     from atomserve_amd.engine.engine import create_engine
     from atomserve_amd.engine.sequence import SamplingParams
 
-    requests, longest, decoded, budget, block = 32, 2048, 128, 512, 16
+    requests, longest, decoded, budget, block = 32, 2048, 128, args.chunk_budget, 16
     max_len = longest + decoded + block
     engine = create_engine(model, EngineConfig(block_size=block, num_blocks=requests * max_len // block,
                                                max_num_seqs=requests, max_num_batched_tokens=budget,
