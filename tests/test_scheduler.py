@@ -263,3 +263,55 @@ def test_windowed_model_gives_pages_back_while_decoding():
                        for x, n in zip(out.seqs, out.num_new_tokens)])  # fmt: skip
         most = max(most, manager.num_blocks - manager.num_free)
     assert q.num_tokens == 23 and most <= 3 and manager.num_free == 6  # 23 tokens never held more than 3 pages
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_arrivals_aborts_and_tight_pools_keep_every_output(seed):
+    """Requests arrive while others run, some are aborted half-way, the pool is small enough to
+    preempt, budgets and row limits are drawn at random, half of the prompts share a prefix: every
+    request that finishes has the tokens it gets alone, nothing is shared unsafely at any step,
+    and every page is back at the end."""
+    import random
+
+    rng = random.Random(seed)
+    bs = rng.choice([2, 4, 8])
+    longest = 40
+    blocks = rng.randint(-(-longest // bs), 2 * -(-longest // bs))
+    seqs_limit = rng.randint(1, 6)
+    config = dict(block_size=bs, num_blocks=blocks, max_model_len=min(longest, blocks * bs), max_num_seqs=seqs_limit,
+                  max_num_batched_tokens=rng.randint(seqs_limit, 24), enable_prefix_caching=rng.random() < 0.7)  # fmt: skip
+    s, runner = make(**config)
+    prefix = [rng.randrange(1, 400) for _ in range(2 * bs + 1)]
+    arrivals = []
+    for i in range(14):
+        own = [rng.randrange(1, 400) for _ in range(rng.randint(1, 20))]
+        prompt = (prefix + own)[: longest - 13] if rng.random() < 0.5 else own
+        params = SamplingParams(temperature=0.0, max_tokens=rng.randint(1, 12), ignore_eos=True)
+        arrivals.append((rng.randint(0, 12), Sequence(i, prompt, params)))
+    aborts = {rng.randrange(14): rng.randint(1, 30) for _ in range(3)}  # request -> step at which it is aborted
+    step, preemptions, aborted = 0, 0, set()
+    while s.has_work or any(at >= step for at, _ in arrivals):
+        for at, seq in arrivals:
+            if at == step:
+                s.add(seq)
+        for victim, at in aborts.items():
+            if at == step and s.abort(victim) is not None:
+                aborted.add(victim)
+        if s.has_work:
+            out = s.schedule()
+            assert out.seqs, "no progress"
+            assert len(out.seqs) <= seqs_limit and out.num_tokens <= config["max_num_batched_tokens"]
+            sharing_is_safe(s)
+            preemptions += len(out.preempted)
+            s.update(out, runner.execute(out))
+            s.manager.check()
+        step += 1
+        assert step < 2000
+    assert s.manager.num_free == blocks
+    for _, seq in arrivals:
+        if seq.id in aborted:
+            assert seq.finish_reason == "abort"
+            continue
+        assert seq.finish_reason == "length"
+        alone_out = run([seq.token_ids[: seq.num_prompt_tokens]], seq.params, block_size=bs)[0][0]
+        assert seq.output_ids == alone_out, (seed, seq.id, preemptions)
