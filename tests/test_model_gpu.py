@@ -69,6 +69,27 @@ def test_mixed_requests_with_pages_used_again(setup, dtype):
     assert replay.manager.num_free == replay.manager.num_blocks
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_traces_in_32_bit(setup, seed):
+    """Requests, portion sizes around the edges of pages and tiles, how many are live and how much
+    of each is prompt drawn at random, the pool as small as the trace allows: in 32-bit every
+    wanted row is the plain model's to a tenth of the bound, so anything a cut or a reused page
+    breaks shows far above rounding."""
+    import random
+
+    name, raw, weights, path, _ = setup
+    rng = random.Random(7 * seed + (name == "B"))
+    longest = min(raw["max_position_embeddings"], rng.choice([40, 130, 250]))
+    requests = {f"r{i}": rc.random_ids(raw["vocab_size"], rng.randint(2, longest), seed=900 + 10 * seed + i)
+                for i in range(rng.randint(2, 7))}  # fmt: skip
+    sizes = tuple(rng.choice([2, 3, 5, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100]) for _ in range(6))
+    steps = rc.mixed(requests, seed=seed, max_live=rng.randint(1, 4), prompt_fraction=rng.choice([0.3, 0.6, 0.95]), sizes=sizes)
+    replay = make_replay(path, "float32", rc.live_token_bound(steps))
+    worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, {})
+    assert rows > 0 and worst <= 0.3 * TOL["float32"] * max(scale, 1.0)
+    assert replay.manager.num_free == replay.manager.num_blocks
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(setup, dtype):
     name, raw, weights, path, cache = setup
