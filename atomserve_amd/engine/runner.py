@@ -15,6 +15,7 @@ from atomserve_amd.cache.manager import CacheManager
 from atomserve_amd.cache.pools import CachePools
 from atomserve_amd.engine.batch import Row, Staging, StepBatch
 from atomserve_amd.engine.sequence import StepResult
+from atomserve_amd.kernels import ops
 from atomserve_amd.sampling.sampler import Sampler
 
 
@@ -84,8 +85,13 @@ class DecodeGraphs:
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 r.model.forward(batch)  # loads every library and warms the allocator before capture
+                for _ in range(3):  # and while the library's products are still being tried, again
+                    if not ops.library_trials_pending():
+                        break
+                    r.model.forward(batch)
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
+            ops.settle_library_choices()  # what the warm-up tried among the library's products is decided now
             batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
             graph = torch.cuda.CUDAGraph()
             # No garbage collection while the stream is capturing: a collected object of an

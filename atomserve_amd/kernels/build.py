@@ -21,7 +21,8 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]  # fmt: skip
 HEADERS = ["common.h"]
-LIBRARIES = ("elementwise", "attention", "gemm", "sampling")
+LIBRARIES = ("elementwise", "attention", "gemm", "sampling", "blas")
+LINK = {"blas": ["-lhipblaslt"]}  # what a library links beside the HIP runtime
 
 
 class BuildError(RuntimeError):
@@ -37,7 +38,7 @@ def _hipcc() -> str:
 
 
 def _source_hash(name: str) -> str:
-    h = hashlib.sha256(" ".join(FLAGS).encode())
+    h = hashlib.sha256(" ".join([*FLAGS, *LINK.get(name, [])]).encode())
     for rel in [f"{name}.hip", *HEADERS]:
         with open(os.path.join(CSRC, rel), "rb") as f:
             h.update(rel.encode())
@@ -79,7 +80,7 @@ def compile_library(name: str, out_dir: str, quiet: bool = False) -> str:
     digest = _source_hash(name)
     target = os.path.join(out_dir, f"lib_{name}.so")
     tmp = f"{target}.{os.getpid()}.tmp"
-    cmd = [_hipcc(), *FLAGS, os.path.join(CSRC, f"{name}.hip"), "-o", tmp]
+    cmd = [_hipcc(), *FLAGS, os.path.join(CSRC, f"{name}.hip"), "-o", tmp, *LINK.get(name, [])]
     if not quiet:
         print(f"atomserve_amd: compiling {name}.hip for {ARCH} ...", file=sys.stderr, flush=True)
     start = time.time()

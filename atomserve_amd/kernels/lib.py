@@ -7,7 +7,7 @@ library cannot be built or loaded raises.
 """
 
 import ctypes
-from ctypes import c_double, c_float, c_int, c_void_p
+from ctypes import c_double, c_float, c_int, c_size_t, c_void_p
 
 import torch  # noqa: F401  (loads libamdhip64 first)
 
@@ -30,6 +30,8 @@ SIGNATURES = {
     "as_gemm_bf16_gated": ("gemm", [P, P, P, I, I, I, P]),
     "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, I, I, I, P]),
     "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, I, I, I, I, P]),
+    "as_blas_plan": ("blas", [I, I, I, I, c_size_t]),
+    "as_blas_gemm": ("blas", [P, P, P, I, I, I, I, I, P, c_size_t, P]),
     "as_argmax": ("sampling", [P, P, I, I, P]),
     "as_sample": ("sampling", [P, I, I, P, P, P, P, P, P, P]),
     "as_sample_split": ("sampling", [P, I, I, P, P, P, P, P, P, P, P, P]),

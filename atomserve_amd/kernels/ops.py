@@ -9,7 +9,7 @@ import math
 
 import torch
 
-from atomserve_amd.kernels.lib import KernelError, call
+from atomserve_amd.kernels.lib import KernelError, call, entry
 
 F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
 _DT = {F32: 0, BF16: 1}
@@ -267,10 +267,102 @@ def gemm(a, w, out) -> None:
         raise KernelError(f"gemm: unsupported output dtype {out.dtype}")
     if _few_rows(M, K, N):
         call("as_gemm_bf16_skinny", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, 0, _stream())
-    elif out.dtype == BF16:
+    else:
+        _library_gemm(a, w, out, M, N, K)
+
+
+# ---- the library's product, called directly -------------------------------------------------
+#
+# hipBLASLt through `csrc/blas.hip` instead of torch.mm: the same kernels for two thirds of the
+# time on the host.  For the row counts of LIBRARY_TUNED_ROWS (decode steps of 17 to 64 requests
+# are padded to these and replayed thousands of times) the library's first candidate is often
+# not its fastest on this GPU, so the first calls of such a shape try the candidates in turn, each
+# on the weights of the layer that happens to call (cold, as every decode step meets them), timed
+# by events in place; when every candidate has run LIBRARY_TRIALS_EACH times (the first run of a
+# kernel is slow), or a capture begins, the fastest stays.
+LIBRARY_WORKSPACE_BYTES = 64 << 20
+LIBRARY_TUNED_ROWS = (32, 64)
+LIBRARY_TRIALS_EACH = 4
+_library = {"workspace": None, "choice": {}, "trials": {}}
+
+
+def _torch_gemm(a, w, out) -> None:
+    if out.dtype == BF16:
         torch.mm(a, w.t(), out=out)
     else:
         out.copy_(torch.mm(a, w.t()))
+
+
+def _library_gemm(a, w, out, M, N, K) -> None:
+    state = _library
+    key = (M, N, K, out.dtype)
+    choice = state["choice"].get(key)
+    if choice is None:
+        capturing = torch.cuda.is_current_stream_capturing()
+        if state["workspace"] is None:
+            if capturing:  # nothing is allocated for good inside a capture: torch's own call this once
+                return _torch_gemm(a, w, out)
+            state["workspace"] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
+        trial = state["trials"].get(key)
+        if trial is None:
+            count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
+            if count == 0 or count == 1 or M not in LIBRARY_TUNED_ROWS:
+                choice = state["choice"][key] = count - 1 if count < 2 else 0
+            else:
+                trial = state["trials"][key] = {"count": count, "runs": []}
+        if trial is not None:
+            if not capturing and len(trial["runs"]) < LIBRARY_TRIALS_EACH * trial["count"]:
+                candidate = len(trial["runs"]) % trial["count"]
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                try:
+                    _library_call(a, w, out, M, N, K, candidate)
+                except KernelError:  # a candidate that does not run: the first one does
+                    trial["runs"].append((candidate, None, None))
+                    return _library_call(a, w, out, M, N, K, 0)
+                end.record()
+                trial["runs"].append((candidate, start, end))
+                return
+            choice = state["choice"][key] = _fastest_of(state["trials"].pop(key))
+    if choice < 0:  # the library offers nothing for this shape through this door
+        return _torch_gemm(a, w, out)
+    _library_call(a, w, out, M, N, K, choice)
+
+
+def _library_call(a, w, out, M, N, K, candidate) -> None:
+    call("as_blas_gemm", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, candidate,
+         _ptr(_library["workspace"]), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip
+
+
+def library_trials_pending() -> bool:
+    """Whether some shape is still trying candidates (a warm-up may then run once more)."""
+    return bool(_library["trials"])
+
+
+def settle_library_choices() -> None:
+    """Ends every trial that is under way, with what has been timed so far.  Called before a capture
+    begins, so that the captured launches are the ones later replays should make."""
+    state = _library
+    if state["trials"]:
+        torch.cuda.current_stream().synchronize()
+        for key in list(state["trials"]):
+            state["choice"][key] = _fastest_of(state["trials"].pop(key))
+
+
+def _fastest_of(trial) -> int:
+    """The candidate whose runs took least on average, among the runs that were timed and have
+    finished and leaving out each candidate's first (which loads the kernel); 0 if none."""
+    times = {}
+    for candidate, start, end in trial["runs"]:
+        if start is not None and end.query():
+            times.setdefault(candidate, []).append(start.elapsed_time(end))
+    best, best_time = 0, float("inf")
+    for candidate, took in times.items():
+        rest = took[1:] or took
+        mean = sum(rest) / len(rest)
+        if mean < best_time:
+            best, best_time = candidate, mean
+    return best
 
 
 GATED_MAX_K = 6144  # the widest input the fused product-and-activation kernel keeps in registers

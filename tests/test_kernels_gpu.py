@@ -264,6 +264,81 @@ def test_gemm_silu_mul_bf16(ops, M, I, K):
     assert close_bf16(out, pk.silu_mul(gate_up))
 
 
+def test_every_candidate_of_the_library_gives_the_product(ops):
+    """Above the few-rows kernels the product is hipBLASLt's, called directly with one of the
+    library's own candidates: each of them is the product, and a shape of a decode bucket settles
+    on one of them after trying them in turn."""
+    from atomserve_amd.kernels.lib import call, entry
+
+    torch.manual_seed(21)
+    workspace = torch.empty(ops.LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=DEV)
+    for M, N, K, dtype in ((64, 520, 1024, BF16), (100, 264, 200, F32), (32, 4096, 4096, BF16)):
+        a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
+        ref = pk.gemm(a, w)
+        count = entry("as_blas_plan")(M, N, K, 0 if dtype == F32 else 1, ops.LIBRARY_WORKSPACE_BYTES)
+        assert count >= 1
+        for candidate in range(count):
+            out = torch.zeros(M, N, dtype=dtype, device=DEV)
+            call("as_blas_gemm", a.data_ptr(), w.data_ptr(), out.data_ptr(), 0 if dtype == F32 else 1, M, N, K, candidate,
+                 workspace.data_ptr(), ops.LIBRARY_WORKSPACE_BYTES, torch.cuda.current_stream().cuda_stream)  # fmt: skip
+            if dtype == BF16:
+                assert close_bf16(out, ref, scale=math.sqrt(K)), (M, N, K, candidate)
+            else:
+                assert torch.allclose(out, ref, atol=math.sqrt(K) * 2.0**-8, rtol=2.0**-7), (M, N, K, candidate)
+        with pytest.raises(ops.KernelError):
+            call("as_blas_gemm", a.data_ptr(), w.data_ptr(), out.data_ptr(), 1, M, N, K, count, workspace.data_ptr(),
+                 ops.LIBRARY_WORKSPACE_BYTES, torch.cuda.current_stream().cuda_stream)  # fmt: skip
+    # 64 rows is a decode bucket: the first calls try the candidates, then one stays
+    M, N, K = 64, 528, 8192
+    a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
+    ref = pk.gemm(a, w)
+    out = torch.empty(M, N, dtype=BF16, device=DEV)
+    for _ in range(ops.LIBRARY_TRIALS_EACH * 16 + 2):
+        out.zero_()
+        ops.gemm(a, w, out)
+        assert close_bf16(out, ref, scale=math.sqrt(K))
+    assert (M, N, K, BF16) in ops._library["choice"]
+    ops.settle_library_choices()  # and whatever other tests left half tried
+    assert not ops.library_trials_pending()
+
+
+def test_library_candidates_replay_from_a_graph(ops):
+    """Each candidate captured once and replayed with other inputs and a workspace full of noise,
+    with eager work and synchronisations between the replays: every replay gives what the eager
+    call gives (a candidate that clears its workspace through a captured memset would not)."""
+    from atomserve_amd.kernels.lib import call, entry
+
+    size = ops.LIBRARY_WORKSPACE_BYTES
+    workspace = torch.empty(size, dtype=torch.uint8, device=DEV)
+    for M, N, K in ((64, 4096, 4096), (32, 4096, 12288), (64, 1024, 3072)):
+        torch.manual_seed(M + K)
+        w = (torch.randn(N, K, device=DEV) * 0.02).to(BF16)
+        a = torch.randn(M, K, device=DEV).to(BF16)
+        out = torch.empty(M, N, dtype=BF16, device=DEV)
+        for candidate in range(entry("as_blas_plan")(M, N, K, 1, size)):
+            def run():
+                call("as_blas_gemm", a.data_ptr(), w.data_ptr(), out.data_ptr(), 1, M, N, K, candidate,
+                     workspace.data_ptr(), size, torch.cuda.current_stream().cuda_stream)  # fmt: skip
+
+            run()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                run()
+            for _ in range(3):
+                a.copy_(torch.randn(M, K, device=DEV).to(BF16))
+                workspace[: 1 << 20].random_(0, 255)
+                out.zero_()
+                graph.replay()
+                torch.cuda.synchronize()
+                replayed = out.clone()
+                workspace[: 1 << 20].random_(0, 255)
+                out.zero_()
+                run()
+                torch.cuda.synchronize()
+                assert torch.equal(replayed, out), (M, N, K, candidate)
+
+
 def test_gemm_silu_mul_fp32(ops):
     torch.manual_seed(10)
     a, w = torch.randn(5, 72, device=DEV), torch.randn(2 * 50, 72, device=DEV) / 8

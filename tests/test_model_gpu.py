@@ -125,13 +125,18 @@ def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
     and synchronisations between them, for row counts in the small buckets (one and two row tiles
     of this package's products) and the large ones (whose matrix products are the library's).  The
     last step's logits are also the plain model's."""
-    from atomserve_amd.cache.manager import CacheManager
-    from atomserve_amd.engine.batch import Row
-    from atomserve_amd.engine.runner import ModelRunner
     from atomserve_amd.weights.loader import load_model
 
     name, raw, weights, path, cache = setup
     model, _, _ = load_model(path, getattr(torch, dtype), "cuda:0")
+    graphs_against_eager(model, raw, weights, dtype, num_requests, torch.float64)
+
+
+def graphs_against_eager(model, raw, weights, dtype, num_requests, plain_dtype):
+    from atomserve_amd.cache.manager import CacheManager
+    from atomserve_amd.engine.batch import Row
+    from atomserve_amd.engine.runner import ModelRunner
+
     vocab = raw["vocab_size"]
     prompts = [rc.random_ids(vocab, 5 + 3 * (i % 11), seed=300 + i) for i in range(num_requests)]
     later = [rc.random_ids(vocab, 12, seed=400 + i) for i in range(num_requests)]  # the tokens decoded, given
@@ -166,9 +171,25 @@ def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
         assert a.shape == b.shape and torch.isfinite(a).all()
         check(float((a - b).abs().max()), float(b.abs().max()), dtype)
     for i in (0, num_requests // 2, num_requests - 1):
-        ref = plain.logits(raw, weights, prompts[i] + later[i][:8])[-1].float()
+        ref = plain.logits(raw, weights, prompts[i] + later[i][:8], dtype=plain_dtype)[-1].float()
         for out in seen.values():
             check(float((out[-1][i] - ref).abs().max()), float(ref.abs().max()), dtype)
+
+
+
+
+def test_decode_graphs_at_real_layer_sizes(tmp_path_factory):
+    """The same at Qwen3-8B's layer sizes, where the products of 17 to 64 rows are the library's
+    with the candidate that the warm-up's trials chose: replays of the captured steps give what
+    eager steps give, replay after replay, and what the plain model gives."""
+    from atomserve_amd.weights.loader import load_model
+
+    raw = {**TINY_B_LIKE_8B}
+    weights = plain_random_weights(raw, seed=78, std=0.02, gain_std=0.1)
+    path = write_model_dir(str(tmp_path_factory.mktemp("real_graphs")), raw, weights, torch.bfloat16)
+    model, _, _ = load_model(path, torch.bfloat16, "cuda:0")
+    for num_requests in (21, 40):
+        graphs_against_eager(model, raw, weights, "bfloat16", num_requests, torch.float32)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
