@@ -312,6 +312,7 @@ def _library_gemm(a, w, out, M, N, K) -> None:
                 trial = state["trials"][key] = {"count": count, "runs": []}
         if trial is not None:
             if not capturing and len(trial["runs"]) < LIBRARY_TRIALS_EACH * trial["count"]:
+                trial["last"] = (a, w, out)
                 candidate = len(trial["runs"]) % trial["count"]
                 start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 start.record()
@@ -323,7 +324,9 @@ def _library_gemm(a, w, out, M, N, K) -> None:
                 end.record()
                 trial["runs"].append((candidate, start, end))
                 return
-            choice = state["choice"][key] = _fastest_of(state["trials"].pop(key))
+            trial = state["trials"].pop(key)
+            trial.pop("last", None)
+            choice = state["choice"][key] = _fastest_of(trial)
     if choice < 0:  # the library offers nothing for this shape through this door
         return _torch_gemm(a, w, out)
     _library_call(a, w, out, M, N, K, choice)
@@ -343,10 +346,25 @@ def settle_library_choices() -> None:
     """Ends every trial that is under way, with what has been timed so far.  Called before a capture
     begins, so that the captured launches are the ones later replays should make."""
     state = _library
-    if state["trials"]:
+    for key in list(state["trials"]):
+        trial = state["trials"].pop(key)
+        # a shape that a pass meets once (the head) has not come round often enough: the rest of
+        # its runs are made here, on the operands of its last call
+        a, w, out = trial.pop("last")
+        M, N, K, _ = key
+        while len(trial["runs"]) < LIBRARY_TRIALS_EACH * trial["count"]:
+            candidate = len(trial["runs"]) % trial["count"]
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            try:
+                _library_call(a, w, out, M, N, K, candidate)
+            except KernelError:
+                trial["runs"].append((candidate, None, None))
+                continue
+            end.record()
+            trial["runs"].append((candidate, start, end))
         torch.cuda.current_stream().synchronize()
-        for key in list(state["trials"]):
-            state["choice"][key] = _fastest_of(state["trials"].pop(key))
+        state["choice"][key] = _fastest_of(trial)
 
 
 def _fastest_of(trial) -> int:
