@@ -329,3 +329,65 @@ def test_command_line_generates(setup, capsys):
                  "--kv-mem-gb", "0.01", "--max-num-seqs", "4", "--max-batched-tokens", "16"]) == 0  # fmt: skip
     out = [js.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
     assert len(out) == 1 and len(out[0]["output_ids"]) <= 4
+
+
+def test_engine_thread_under_concurrent_clients(setup):
+    """Two seconds of serving on the engine's own thread: clients on eight threads submit prompts
+    of all lengths (some share a prefix), stream, and abort now and then, with a pool small
+    enough to preempt.  Every request ends as asked or aborted, with as many tokens as it asked
+    for; nothing is left running and every page is back."""
+    import random
+    import threading
+    import time
+
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.weights import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, torch.bfloat16, "cuda:0")
+    limit = min(raw["max_position_embeddings"], 200)
+    engine = create_engine(model, EngineConfig(block_size=16, num_blocks=40, max_num_seqs=6, max_num_batched_tokens=48,
+                                               max_model_len=limit), seed=0)  # fmt: skip
+    engine.start()
+    stop = time.time() + 2.0
+    counts = {"length": 0, "abort": 0}
+    problems = []
+    lock = threading.Lock()
+
+    def client(i):
+        rng = random.Random(i)
+        shared = rc.random_ids(raw["vocab_size"], 33, seed=1)
+        while time.time() < stop:
+            prompt = (shared if rng.random() < 0.4 else []) + rc.random_ids(raw["vocab_size"], rng.randint(1, 90), seed=rng.randrange(1 << 30))
+            params = SamplingParams(temperature=rng.choice([0.0, 0.8]), max_tokens=rng.randint(1, 40), ignore_eos=True)
+            try:
+                handle = engine.submit(prompt, params)
+                cut = rng.randint(1, 10) if rng.random() < 0.25 else None
+                got = 0
+                for _ in handle:
+                    got += 1
+                    if got == cut:
+                        handle.abort()
+                with lock:
+                    counts[handle.finish_reason] += 1
+                    if handle.finish_reason == "length" and got != params.max_tokens:
+                        problems.append(f"{got} tokens for max_tokens {params.max_tokens}")
+            except Exception as e:  # noqa: BLE001  (reported below, on the main thread)
+                with lock:
+                    problems.append(repr(e))
+                return
+
+    threads = [threading.Thread(target=client, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=60)
+    assert not any(t.is_alive() for t in threads), "a client never got its last token"
+    time.sleep(0.2)
+    stats = engine.stats()
+    engine.shutdown()
+    assert not problems, problems[:3]
+    assert counts["length"] > 20 and counts["abort"] > 0
+    assert stats["running"] == stats["waiting"] == stats["kv_blocks_used"] == 0
