@@ -25,6 +25,7 @@ from atomserve_amd.config.engine_config import EngineConfig
 from atomserve_amd.engine.runner import ModelRunner
 from atomserve_amd.engine.scheduler import Scheduler
 from atomserve_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus
+from atomserve_amd.kernels import ops
 
 
 @dataclass
@@ -223,4 +224,6 @@ def create_engine(model, engine_config: EngineConfig, eos_token_ids=frozenset(),
     manager = CacheManager(model.cache_requests(), engine_config.block_size, engine_config.num_blocks,
                            engine_config.max_num_seqs)  # fmt: skip
     runner = ModelRunner(model, manager)
+    if runner.device.type == "cuda":
+        ops.tune_library_rows(engine_config.max_num_batched_tokens)  # what a step with a prompt's portion brings
     return Engine(runner, Scheduler(engine_config, eos_token_ids, manager), seed=seed)

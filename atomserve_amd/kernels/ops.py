@@ -281,7 +281,7 @@ def gemm(a, w, out) -> None:
 # by events in place; when every candidate has run LIBRARY_TRIALS_EACH times (the first run of a
 # kernel is slow), or a capture begins, the fastest stays.
 LIBRARY_WORKSPACE_BYTES = 64 << 20
-LIBRARY_TUNED_ROWS = (32, 64)
+LIBRARY_TUNED_ROWS = {32, 64}
 LIBRARY_TRIALS_EACH = 4
 _library = {"workspace": None, "choice": {}, "trials": {}}
 
@@ -335,6 +335,12 @@ def _library_gemm(a, w, out, M, N, K) -> None:
 def _library_call(a, w, out, M, N, K, candidate) -> None:
     call("as_blas_gemm", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, candidate,
          _ptr(_library["workspace"]), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip
+
+
+def tune_library_rows(rows: int) -> None:
+    """Also try the candidates for products of this many rows: a row count that comes again and
+    again, like the token budget of the steps that carry a portion of a prompt."""
+    LIBRARY_TUNED_ROWS.add(int(rows))
 
 
 def library_trials_pending() -> bool:
