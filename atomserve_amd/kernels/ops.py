@@ -177,6 +177,8 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
             limit = 2048
         while part_size < span and groups * math.ceil(span / part_size) > limit:
             part_size *= 2
+        if mfma and groups >= ATTN_FILL_GROUPS:
+            part_size = max(part_size, -(-span // 32) * 32)  # enough workgroups without partitions: no merge
     if mfma and part_size % 32:
         raise KernelError("attention: partitions of the matrix-core kernel are multiples of 32 keys")
     P = max(1, math.ceil(max_context / part_size))
@@ -195,6 +197,7 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
+ATTN_FILL_GROUPS = 512  # (token, kv head) pairs that occupy every compute unit twice over
 PREFILL_MAX_HEAD_DIM = 256  # four stages of 32 keys and values of such heads fill 128 KB of LDS
 
 
