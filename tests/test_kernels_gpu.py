@@ -526,6 +526,20 @@ def test_attention_of_a_decode_step_needs_no_maps(ops, dtype):
         ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables[:3], b, D**-0.5, 0, max(lens))
 
 
+def test_attention_of_a_batch_that_fills_the_gpu(ops):
+    """64 requests of 8 kv heads are 512 workgroups already: the contexts are not partitioned (no
+    merge), each workgroup walks its whole context, of very different lengths."""
+    H, KV, D, bs = 16, 8, 64, 16
+    lens = [1 + (37 * i * i) % 1400 for i in range(64)]
+    assert 64 * KV >= ops.ATTN_FILL_GROUPS
+    q, k_pages, v_pages, tables, positions = paged_case(BF16, H, KV, D, bs, lens, seed=5, k_scale=1.0)
+    out = torch.zeros(64, H, D, dtype=BF16, device=DEV)
+    ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables, out, D**-0.5, 0, max(lens))
+    rows = i32(list(range(64)))
+    ref = pk.paged_attention(q, k_pages, v_pages, rows, positions, rows, tables, D**-0.5)
+    assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2)
+
+
 def test_attention_serves_only_the_listed_tokens(ops):
     """Items select tokens; several tokens of one request share a table and see keys up to
     their own position only."""
