@@ -309,28 +309,19 @@ def _library_gemm(a, w, out, M, N, K) -> None:
         trial = state["trials"].get(key)
         if trial is None:
             count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
-            if count == 0 or count == 1 or M not in LIBRARY_TUNED_ROWS:
-                choice = state["choice"][key] = count - 1 if count < 2 else 0
+            if count == 0:
+                choice = state["choice"][key] = -1  # the library offers nothing for this shape through this door
+            elif count == 1 or M not in LIBRARY_TUNED_ROWS:
+                choice = state["choice"][key] = 0  # the library's first candidate, which is what torch.mm runs
             else:
                 trial = state["trials"][key] = {"count": count, "runs": []}
         if trial is not None:
-            if not capturing and len(trial["runs"]) < LIBRARY_TRIALS_EACH * trial["count"]:
+            if not capturing and not _tried_enough(trial):
                 trial["last"] = (a, w, out)
-                candidate = len(trial["runs"]) % trial["count"]
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-                try:
-                    _library_call(a, w, out, M, N, K, candidate)
-                except KernelError:  # a candidate that does not run: the first one does
-                    trial["runs"].append((candidate, None, None))
-                    return _library_call(a, w, out, M, N, K, 0)
-                end.record()
-                trial["runs"].append((candidate, start, end))
+                _trial_run(trial, a, w, out, M, N, K)
                 return
-            trial = state["trials"].pop(key)
-            trial.pop("last", None)
-            choice = state["choice"][key] = _fastest_of(trial)
-    if choice < 0:  # the library offers nothing for this shape through this door
+            choice = state["choice"][key] = _fastest_of(state["trials"].pop(key))
+    if choice < 0:
         return _torch_gemm(a, w, out)
     _library_call(a, w, out, M, N, K, choice)
 
@@ -338,6 +329,25 @@ def _library_gemm(a, w, out, M, N, K) -> None:
 def _library_call(a, w, out, M, N, K, candidate) -> None:
     call("as_blas_gemm", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, candidate,
          _ptr(_library["workspace"]), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip
+
+
+def _tried_enough(trial) -> bool:
+    return len(trial["runs"]) >= LIBRARY_TRIALS_EACH * trial["count"]
+
+
+def _trial_run(trial, a, w, out, M, N, K) -> None:
+    """Computes the product with the candidate whose turn it is, between two events."""
+    candidate = len(trial["runs"]) % trial["count"]
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    try:
+        _library_call(a, w, out, M, N, K, candidate)
+    except KernelError:  # a candidate that does not run; the first one does
+        trial["runs"].append((candidate, None, None))
+        _library_call(a, w, out, M, N, K, 0)
+        return
+    end.record()
+    trial["runs"].append((candidate, start, end))
 
 
 def tune_library_rows(rows: int) -> None:
@@ -352,26 +362,16 @@ def library_trials_pending() -> bool:
 
 
 def settle_library_choices() -> None:
-    """Ends every trial that is under way, with what has been timed so far.  Called before a capture
-    begins, so that the captured launches are the ones later replays should make."""
+    """Ends every trial that is under way.  Called before a capture begins, so that the captured
+    launches are the ones later replays should make.  A shape that a pass meets once (the head)
+    has not come round often enough by then: the rest of its runs are made here, on the operands
+    of its last call."""
     state = _library
     for key in list(state["trials"]):
         trial = state["trials"].pop(key)
-        # a shape that a pass meets once (the head) has not come round often enough: the rest of
-        # its runs are made here, on the operands of its last call
-        a, w, out = trial.pop("last")
-        M, N, K, _ = key
-        while len(trial["runs"]) < LIBRARY_TRIALS_EACH * trial["count"]:
-            candidate = len(trial["runs"]) % trial["count"]
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            try:
-                _library_call(a, w, out, M, N, K, candidate)
-            except KernelError:
-                trial["runs"].append((candidate, None, None))
-                continue
-            end.record()
-            trial["runs"].append((candidate, start, end))
+        a, w, out = trial["last"]
+        while not _tried_enough(trial):
+            _trial_run(trial, a, w, out, *key[:3])
         torch.cuda.current_stream().synchronize()
         state["choice"][key] = _fastest_of(trial)
 
