@@ -227,6 +227,62 @@ __device__ int block_topk(const float* __restrict__ x, int V, int k, unsigned lo
   return found;
 }
 
+// The order-preserving bits of the k-th largest value of a row (1 <= k <= number of usable
+// entries, else of the smallest usable one), by radix selection over ALL entries: four passes,
+// eight bits each.  For a k beyond what block_topk holds; the caller keeps every entry whose bits
+// are at least the result, so entries equal to the k-th stay together.  0 if nothing is usable.
+__device__ unsigned int block_kth_value_bits(const float* __restrict__ x, int V, int k, TopKShared& sh) {
+  const int tid = threadIdx.x, T = blockDim.x;
+  int usable = 0;
+  for (int i = tid; i < V; i += T) usable += x[i] == x[i];
+  __syncthreads();
+  if (tid == 0) sh.count = 0;
+  __syncthreads();
+  if (usable) atomicAdd(&sh.count, (unsigned int)usable);
+  __syncthreads();
+  const int have = (int)sh.count;
+  if (have == 0) return 0u;
+  unsigned int prefix = 0, mask = 0;
+  int want = k < have ? k : have;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    if (tid < 256) sh.hist[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < V; i += T) {
+      const unsigned long long key = make_key(x[i], i);
+      const unsigned int bits = (unsigned int)(key >> 32);
+      if (key != 0ull && (bits & mask) == prefix) atomicAdd(&sh.hist[(bits >> shift) & 255], 1u);
+    }
+    __syncthreads();
+    // the bin with (entries in higher bins) < want <= (entries in this bin and higher): as in block_topk
+    int above_incl = 0, own = 0;
+    if (tid < 256) {
+      own = (int)sh.hist[tid];
+      above_incl = own;
+      const int lane = tid & 63;
+#pragma unroll
+      for (int off = 1; off < WAVE; off <<= 1) {
+        const int o = __shfl_down(above_incl, off, WAVE);
+        if (lane + off < WAVE) above_incl += o;
+      }
+      if (lane == 0) sh.wave_total[tid >> 6] = above_incl;
+    }
+    __syncthreads();
+    if (tid < 256) {
+      for (int w = (tid >> 6) + 1; w < 4; ++w) above_incl += sh.wave_total[w];
+      const int above = above_incl - own;
+      if (above < want && above_incl >= want) {
+        sh.prefix = prefix | ((unsigned int)tid << shift);
+        sh.remaining = want - above;
+      }
+    }
+    __syncthreads();
+    prefix = sh.prefix;
+    want = sh.remaining;
+    mask |= 255u << shift;
+  }
+  return prefix;
+}
+
 // ---- greedy -----------------------------------------------------------------------
 __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(const float* __restrict__ logits,
                                                                 int* __restrict__ out, int V) {
@@ -277,9 +333,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int counter = counters[row];
   if (T <= 0.f || p_keep <= 0.f) { k = 1; T = 1.f; }  // greedy: the best token alone
   const bool all = (k <= 0 || k >= V);
+  const bool wide = !all && k > SAMPLE_KMAX;  // more candidates than LDS ranks: a floor on the value instead
 
-  if (!all) {
-    if (k > SAMPLE_KMAX) k = SAMPLE_KMAX;  // refused on the host; never index outside
+  if (!all && !wide) {
     const int found = block_topk(x, V, k, sel, topk_shared);
     __syncthreads();
     if (tid == 0) {
@@ -306,15 +362,18 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     return;
   }
 
-  // Every token is a candidate.  With p_i = softmax(x / T)_i, argmax p_i / E_i equals
-  // argmax x_i / T - log E_i, so no normalisation is needed for the draw itself.
+  // Every token is a candidate (or, with a top-k beyond SAMPLE_KMAX, every token whose logit is at
+  // least the k-th largest: equal ones stay together).  With p_i = softmax(x / T)_i, argmax p_i / E_i
+  // equals argmax x_i / T - log E_i, so no normalisation is needed for the draw itself.
+  const unsigned int floor_bits = wide ? block_kth_value_bits(x, V, k, topk_shared) : 0u;
+  auto usable = [&](float v, int i) { return v == v && (!wide || (unsigned int)(make_key(v, i) >> 32) >= floor_bits); };
   float keep_from = -1.f;  // tokens with p_i >= keep_from stay
   float mx = -__builtin_inff();
   for (int i = tid; i < V; i += SAMPLE_THREADS) { const float v = x[i]; if (v == v) mx = fmaxf(mx, v); }
   mx = block_max_f32(mx, fred);
   float z = 0.f;
   if (p_keep < 1.f) {
-    for (int i = tid; i < V; i += SAMPLE_THREADS) { const float v = x[i]; if (v == v) z += expf((v - mx) / T); }
+    for (int i = tid; i < V; i += SAMPLE_THREADS) { const float v = x[i]; if (usable(v, i)) z += expf((v - mx) / T); }
     z = block_sum(z, fred);
     // Bisection for the smallest probability that is still kept: a token stays iff the mass
     // of the tokens above it is below top_p.  f(t) = mass of tokens with p > t falls with t;
@@ -326,7 +385,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       float mass = 0.f;
       for (int i = tid; i < V; i += SAMPLE_THREADS) {
         const float v = x[i];
-        if (v == v) { const float p = expf((v - mx) / T) / z; if (p > mid) mass += p; }
+        if (usable(v, i)) { const float p = expf((v - mx) / T) / z; if (p > mid) mass += p; }
       }
       mass = block_sum(mass, fred);
       if (mass >= p_keep) lo = mid; else hi = mid;
@@ -336,7 +395,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   unsigned long long best = 0ull;
   for (int i = tid; i < V; i += SAMPLE_THREADS) {
     const float v = x[i];
-    if (v != v) continue;
+    if (!usable(v, i)) continue;
     if (keep_from > 0.f && expf((v - mx) / T) / z < keep_from && v < mx) continue;  // the best always stays
     const unsigned long long key = make_key(v / T - logf(exp1_noise(seed, counter, i)), i);
     best = key > best ? key : best;

@@ -490,8 +490,9 @@ def sample(logits, temperature, top_k, top_p, seeds, counters, out, max_top_k=No
     """One token per row: top-k (0: all), temperature (0: greedy), top-p, seeded draw.
 
     temperature, top_p fp32 [B]; top_k, counters int32 [B]; seeds int64 [B]; out int32 [B].
-    top_k values must be 0 (or >= vocabulary) or at most SAMPLE_MAX_TOP_K; checked by the caller
-    on the host values it uploads.  max_top_k: the caller's promise that every row keeps between 1
+    A top_k of 0 (or >= vocabulary) keeps all tokens; up to SAMPLE_MAX_TOP_K the candidates are
+    ranked (the lower index first among equals); beyond, every token at least as large as the k-th
+    largest stays (equal ones together).  max_top_k: the caller's promise that every row keeps between 1
     and this many candidates (a greedy row keeps 1); up to SAMPLE_SPLIT_MAX_TOP_K the rows are
     then searched by many workgroups each, with the same result."""
     _check(logits, "logits", F32, (None, None))

@@ -41,10 +41,9 @@ class Sampler:
         top_k, kept = [], []
         for p in params:
             k = p.top_k if 0 < p.top_k < vocab else 0
-            if k > ops.SAMPLE_MAX_TOP_K:
-                raise ValueError(f"top_k {k} is beyond the kernel's {ops.SAMPLE_MAX_TOP_K}; use 0 for all tokens")
             top_k.append(k)
-            # candidates the row keeps; all tokens (k == 0) is left to the one-workgroup kernel
+            # candidates the row keeps; all tokens (k == 0) and more than the kernels rank in LDS
+            # are left to the one-workgroup kernel
             kept.append(1 if p.temperature <= 0 or p.top_p <= 0 else (k or ops.SAMPLE_MAX_TOP_K + 1))
         # One upload: int32 rows (temperature and top_p as their bit patterns, top_k, tokens sampled
         # so far), then the 64-bit seeds.

@@ -79,6 +79,30 @@ def test_greedy_and_sampled_rows_mix_in_one_batch(sampler, seed):
     assert sampler.sample(logits, batch) == [1, 2]
 
 
-def test_too_wide_a_top_k_is_refused(sampler):
-    with pytest.raises(ValueError, match="top_k"):
-        sampler.sample(torch.zeros(1, 5000, device=DEV), seqs(1, temperature=1.0, top_k=2000))
+def test_top_k_beyond_what_is_ranked_keeps_the_k_largest(sampler):
+    """A top-k of thousands is a floor on the logit (the k-th largest, found over the whole row):
+    draws come from those k tokens only, with the plain distribution's frequencies, also with a
+    top-p on top."""
+    from tests import plain_qwen3 as plain
+
+    torch.manual_seed(3)
+    V, k, n = 6000, 2500, 3000
+    row = torch.randn(V) * 0.7
+    row[torch.randperm(V)[:5]] += 3.0  # a few likely tokens, so that frequencies can be compared
+    logits = row.repeat(n, 1).to(DEV)
+    for top_p in (1.0, 0.9):
+        batch = seqs(n, temperature=1.0, top_k=k, top_p=top_p)
+        got = torch.tensor(sampler.sample(logits, batch))
+        dist = plain.sampling_distribution(row, 1.0, k, top_p)
+        assert bool((dist[got] > 0).all()), "a token outside the k largest (or the top-p set) was drawn"
+        dist = dist / dist.sum()
+        top = dist.topk(5).indices
+        freq = torch.bincount(got, minlength=V)[top].double() / n
+        sigma = (dist[top] * (1 - dist[top]) / n).sqrt()
+        assert bool(((freq - dist[top]).abs() <= 5 * sigma).all()), (freq, dist[top])
+    # the k-th largest has equals: they all stay (k = 1100 reaches into a run of equal logits)
+    tied = torch.full((V,), -2.0)
+    tied[:1000] = torch.linspace(3.0, 1.0, 1000)
+    tied[1000:1400] = 0.5  # 400 equal logits across the k-th place
+    got = set(sampler.sample(tied.repeat(4000, 1).to(DEV), seqs(4000, temperature=2.0, top_k=1100, top_p=1.0)))
+    assert max(got) < 1400 and len([t for t in got if t >= 1100]) > 0
