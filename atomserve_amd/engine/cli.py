@@ -128,6 +128,7 @@ def main(argv=None) -> int:
     engine_config = engine_config_for(args, block_bytes, model.plan.max_positions)
     engine = create_engine(model, engine_config, eos_ids(model_dir), seed=args.seed)
     engine.generate([[0]], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))  # compile and warm up
+    engine.warm_up()  # and capture the decode steps of every batch size now, not at their first use
     print(
         f"Ready in {time.perf_counter() - start:.1f}s. KV cache: "
         f"{engine_config.num_blocks * engine_config.block_size:,} tokens, context up to {engine_config.max_model_len:,}.",

@@ -132,6 +132,15 @@ class Engine:
             pass
         return [list(h) for h in handles]
 
+    def warm_up(self) -> int:
+        """Before serving: the decode steps of every batch size up to max_num_seqs are captured now
+        (kernels are compiled and loaded, the library's candidates tried) rather than at their
+        first use.  Returns the number of graphs captured; 0 where decode steps run uncaptured."""
+        graphs = getattr(self.runner, "decode_graphs", None)
+        if graphs is None:
+            return 0
+        return graphs.capture_ahead(self.scheduler.config.max_num_seqs)
+
     def stats(self) -> dict:
         s = self.scheduler
         total = s.manager.num_blocks

@@ -119,6 +119,21 @@ class DecodeGraphs:
         return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)] if wanted else logits[:0]
 
 
+    @torch.inference_mode()
+    def capture_ahead(self, max_rows: int) -> int:
+        """Captures the decode step of every row bucket up to the one that holds `max_rows`, for the
+        first context bucket, with rows that store nothing: a server does this once at its start
+        instead of pausing when a bucket is first met.  Returns how many graphs were captured."""
+        if not self.eligible([Row([0], 0, self.filler_tables, [0], -1, store=False)]):
+            return 0
+        before = len(self.graphs)
+        for n in self.ROW_BUCKETS:
+            self.run([Row([0], 0, self.filler_tables, [0], -1, store=False) for _ in range(n)])
+            if n >= max_rows:
+                break
+        return len(self.graphs) - before
+
+
 class ModelRunner:
     """Owns the model, the cache pools and the sampler; executes one step for a list of rows."""
 

@@ -391,3 +391,23 @@ def test_engine_thread_under_concurrent_clients(setup):
     assert not problems, problems[:3]
     assert counts["length"] > 20 and counts["abort"] > 0
     assert stats["running"] == stats["waiting"] == stats["kv_blocks_used"] == 0
+
+
+def test_warm_up_captures_the_decode_steps_ahead(setup):
+    """After `warm_up` the decode steps of every batch size up to max_num_seqs replay from graphs
+    that are already there, and generation gives the plain model's tokens."""
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.weights import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, torch.float32, "cuda:0")
+    engine = create_engine(model, EngineConfig(block_size=16, num_blocks=64, max_model_len=128, max_num_seqs=6))
+    assert engine.warm_up() == 4  # buckets of 1, 2, 4 and 8 rows
+    graphs = engine.runner.decode_graphs.graphs
+    assert sorted(graphs) == [(n, 1024) for n in (1, 2, 4, 8)] and engine.warm_up() == 0
+    prompts = [rc.random_ids(raw["vocab_size"], n, seed=700 + n) for n in (3, 11, 20, 7, 5)]
+    got = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
+    assert got == [plain.greedy(raw, weights, p, 6) for p in prompts]
+    assert len(graphs) == 4 and engine.stats()["kv_blocks_used"] == 0
