@@ -90,6 +90,36 @@ def test_random_traces_in_32_bit(setup, seed):
     assert replay.manager.num_free == replay.manager.num_blocks
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Every size and option of the configuration drawn anew (head widths in steps of 16 up to 256,
+    groups that are no power of two, one kv head, widths from 24 to 520, an odd vocabulary, one to
+    four layers, eps, theta, tied or not): whole, decoded, in portions and mixed, in both precisions.
+    The matrices shrink with the width so that scores and logits stay of order one to ten."""
+    import random
+
+    rng = random.Random(seed)
+    kv, group, h = rng.choice([1, 2, 3, 4, 5]), rng.choice([1, 2, 3, 4, 5, 6, 7, 8]), rng.choice([24, 40, 56, 72, 88, 104, 136, 200, 264, 520])
+    raw = dict(TINY["A"], vocab_size=rng.choice([50, 97, 1031, 5003]), hidden_size=h,
+               intermediate_size=rng.choice([32, 48, 72, 100, 264, 2 * rng.randint(8, 300)]),
+               num_hidden_layers=rng.randint(1, 4), num_attention_heads=kv * group, num_key_value_heads=kv,
+               head_dim=16 * rng.randint(1, 16), rms_norm_eps=rng.choice([1e-6, 1e-5, 1e-3]),
+               rope_theta=rng.choice([1e4, 5e5, 1e6]), tie_word_embeddings=rng.random() < 0.5,
+               max_position_embeddings=512)  # fmt: skip
+    weights = plain_random_weights(raw, seed=seed + 7, std=min(0.2, 1.0 / h**0.5), gain_std=0.2)
+    path = write_model_dir(str(tmp_path / "drawn"), raw, weights, torch.bfloat16)
+    requests = {f"r{i}": rc.random_ids(raw["vocab_size"], rng.randint(34, 150), seed=seed * 10 + i) for i in range(4)}
+    first = next(iter(requests.items()))
+    cases = [rc.whole(*first), rc.prefill_then_decode(*first), rc.portions(*first), rc.mixed(requests, seed=seed)]
+    cache = {}
+    for dtype in ("float32", "bfloat16"):
+        for steps in cases:
+            replay = make_replay(path, dtype, rc.live_token_bound(steps))
+            worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
+            assert rows > 0 and replay.manager.num_free == replay.manager.num_blocks
+            check(worst, scale, dtype)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(setup, dtype):
     name, raw, weights, path, cache = setup
