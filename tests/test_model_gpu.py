@@ -208,6 +208,46 @@ def graphs_against_eager(model, raw, weights, dtype, num_requests, plain_dtype):
 
 
 
+def test_captured_steps_are_dropped_and_captured_again(setup):
+    """Only so many captured steps are kept.  Three groups of requests (one, three and six rows:
+    three buckets) decode in turn with room for two captured steps, so every step finds its own
+    dropped, captures it again from the shared memory pool and replays it: the logits are those of
+    eager steps throughout."""
+    from atomserve_amd.cache.manager import CacheManager
+    from atomserve_amd.engine.batch import Row
+    from atomserve_amd.engine.runner import ModelRunner
+    from atomserve_amd.weights.loader import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, torch.float32, "cuda:0")
+    vocab = raw["vocab_size"]
+    groups = [[rc.random_ids(vocab, 7 + 5 * i + j, seed=600 + 10 * i + j) for j in range(n)] for i, n in enumerate((1, 3, 6))]
+    seen = {}
+    for use_graphs in (True, False):
+        manager = CacheManager(model.cache_requests(), 16, 64, 16)
+        runner = ModelRunner(model, manager, use_graphs=use_graphs)
+        if use_graphs:
+            runner.decode_graphs.MAX_GRAPHS = 2
+        out = []
+        live = [[[manager.new_request(), 0] for _ in group] for group in groups]
+        for turn in range(5):
+            for group, states in zip(groups, live):
+                rows = []
+                for ids, state in zip(group, states):
+                    tokens = ids[:-4] if turn == 0 else [ids[len(ids) - 5 + turn]]
+                    assert manager.reserve(state[0], state[1], len(tokens))
+                    rows.append(Row(tokens, state[1], state[0].tables, [len(tokens) - 1], -1))
+                    state[1] += len(tokens)
+                out.append(runner.step(rows).float().cpu())
+                if use_graphs:
+                    assert len(runner.decode_graphs.graphs) <= 2
+        seen[use_graphs] = out
+    for a, b in zip(seen[True], seen[False]):
+        check(float((a - b).abs().max()), float(b.abs().max()), "float32")
+    ref = plain.logits(raw, weights, groups[2][5])[-1].float()
+    check(float((seen[True][-1][5] - ref).abs().max()), float(ref.abs().max()), "float32")
+
+
 def test_decode_graphs_at_real_layer_sizes(tmp_path_factory):
     """The same at Qwen3-8B's layer sizes, where the products of 17 to 64 rows are the library's
     with the candidate that the warm-up's trials chose: replays of the captured steps give what
