@@ -81,9 +81,9 @@ class DecodeGraphs:
         longest = max(row.start + 1 for row in rows)
         context = -(-longest // self.CONTEXT_STEP) * self.CONTEXT_STEP
         width = -(-context // bs)
-        padded = [Row(row.tokens, row.start, row.tables, [0], row.state_slot) for row in rows] + [
-            Row([0], 0, self.filler_tables, [0], -1, store=False) for _ in range(n - len(rows))
-        ]
+        # every row of the captured step yields logits; rows that want none are dropped after the replay
+        padded = [row if row.want else Row(row.tokens, row.start, row.tables, [0], row.state_slot) for row in rows]
+        padded += [Row([0], 0, self.filler_tables, [0], -1, store=False) for _ in range(n - len(rows))]
         key = (n, context)
         entry = self.graphs.get(key)
         if entry is not None:

@@ -148,7 +148,7 @@ class Scheduler:
     def _finish_reason(self, seq: Sequence, token: int):
         if token in self.eos_token_ids and not seq.params.ignore_eos:
             return "stop"
-        if len(seq.output_ids) >= seq.params.max_tokens:
+        if seq.num_output_tokens >= seq.params.max_tokens:
             return "length"
         if seq.num_tokens >= self.config.max_model_len:
             return "length"
@@ -157,7 +157,7 @@ class Scheduler:
     def _adopt_prefix(self, seq: Sequence) -> None:
         covered = self.manager.adopt_cached_prefix(seq.cache, seq.token_ids)
         seq.num_computed_tokens = covered
-        if not seq.output_ids:  # count hits on the prompt, not on recomputing a preempted reply
+        if not seq.num_output_tokens:  # count hits on the prompt, not on recomputing a preempted reply
             seq.num_cached_tokens = covered
 
     def _preempt(self, seq: Sequence) -> None:

@@ -67,7 +67,12 @@ class Sequence:
         return len(self.token_ids)
 
     @property
+    def num_output_tokens(self) -> int:
+        return len(self.token_ids) - self.num_prompt_tokens
+
+    @property
     def output_ids(self) -> list:
+        """A copy of the generated tokens; `num_output_tokens` counts them without one."""
         return self.token_ids[self.num_prompt_tokens :]
 
     @property

@@ -51,7 +51,7 @@ class Sampler:
         host[0:B].view(np.float32)[:] = [max(p.temperature, 0.0) for p in params]
         host[B : 2 * B].view(np.float32)[:] = [p.top_p for p in params]
         host[2 * B : 3 * B] = top_k
-        host[3 * B : 4 * B] = [len(s.output_ids) for s in seqs]
+        host[3 * B : 4 * B] = [s.num_output_tokens for s in seqs]
         host[4 * B :].view(np.int64)[:] = [_as_int64(s.noise_seed) for s in seqs]
         dev = torch.from_numpy(host).to(self.device, non_blocking=True)
         floats, ints = dev[: 2 * B].view(torch.float32), dev[2 * B : 4 * B]
