@@ -14,6 +14,7 @@
 // through LDS, partitions by attn_reduce.  Serves fp32 (every row) and bf16 (decode).
 // Plain reference: reference atomserve/kernels.py:167-334, atomserve/model.py:269-289.
 #include "common.h"
+#include <type_traits>
 
 #define NEG_INF (-__builtin_inff())
 
@@ -290,15 +291,45 @@ __device__ __forceinline__ void load_kv_step(KVStep<DC>& st, const bf16* __restr
   }
 }
 
-template <int DC>  // D / 32
+// FRESH: the kernel takes the projection's output qkv [T, H + 2 KV, D] instead of finished queries
+// and does what the norm-rotate-store kernel does before a decode step, for a step whose tokens
+// are their own rows: each workgroup norms and rotates the queries of its group in registers (the
+// partner i + D/2 of coordinate i lies in the same lane when D % 64 == 0), and the workgroup whose
+// partition holds the token's own position makes the token's key and value, writes them to the
+// pages and attends them from LDS, so nothing waits for those writes.  Same arithmetic as
+// qk_norm_rope_store_bf16x8_kernel; the squares are summed in another order.
+struct FreshQKV {
+  const bf16* qkv;
+  const void* qw;      // gains of the per-head norms, D values each, bf16 or fp32
+  const void* kw;
+  const float2* cs;    // [T, D/2] cos, sin of the whole head's rotation
+  const int* slots;    // [T] page * block_size + offset of the new token, -1: keep it out of the pages
+  bf16* k_store;       // the pages again, to write through
+  bf16* v_store;
+  float eps;
+  int store;           // 0: queries only, the pages already hold the token's key and value
+};
+
+__device__ __forceinline__ void load_gains8(const float* w, float* g) {
+  const float4 a = *reinterpret_cast<const float4*>(w), b = *reinterpret_cast<const float4*>(w + 4);
+  g[0] = a.x; g[1] = a.y; g[2] = a.z; g[3] = a.w; g[4] = b.x; g[5] = b.y; g[6] = b.z; g[7] = b.w;
+}
+__device__ __forceinline__ void load_gains8(const bf16* w, float* g) {
+  const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(w);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g[j] = (float)v[j];
+}
+
+template <int DC, int FRESH>  // D / 32; FRESH 0: finished queries, 1: qkv with bf16 gains, 2: with fp32 gains
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ items, const int* __restrict__ positions, const int* __restrict__ tok_row,
     const int* __restrict__ block_tables, int table_width, bf16* __restrict__ out, float* __restrict__ part_m,
     float* __restrict__ part_l, float* __restrict__ part_acc, int H, int KV, int bs, float scale, int window,
-    int part_size, int P) {
+    int part_size, int P, FreshQKV fresh) {
   constexpr int D = DC * 32, DT = DC * 2;  // DT: tiles of 16 output coordinates
   extern __shared__ float smem[];          // [4][16] m, [4][16] l, [4][D][G] acc
+  __shared__ __align__(16) bf16 fresh_kv[2][256];  // FRESH: the new token's key and value
   const int G = H / KV;
   const int item = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
   const int t = items ? items[item] : item;  // null: every token, in order
@@ -322,25 +353,150 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   }
   const int* table = block_tables + (size_t)(tok_row ? tok_row[t] : t) * table_width;  // null: token t is row t
 
+  // Everything is asked for before anything is waited for: the queries (FRESH: as the projection
+  // left them, with the gains and angles of this lane's coordinates; in the workgroup that holds the
+  // token's own position, wave 0 the new key and wave 1 the new value), then the first keys and values.
+  constexpr int HC = DC / 2, HALF = D / 2, PAIRS = (HALF + WAVE - 1) / WAVE;
+  using W = typename std::conditional<FRESH == 2, float, bf16>::type;  // the gains' type
   bf16x8_t qop[DC];
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const size_t row = (size_t)t * (H + 2 * KV);  // FRESH: the token's heads in qkv
   {
-    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bf16* qrow = q + ((size_t)t * H + h0 + min(col, G - 1)) * D + grp * 8;
+    const bf16* qrow = FRESH ? fresh.qkv + (row + h0 + min(col, G - 1)) * D + grp * 8
+                             : q + ((size_t)t * H + h0 + min(col, G - 1)) * D + grp * 8;
 #pragma unroll
     for (int c = 0; c < DC; ++c) qop[c] = col < G ? *reinterpret_cast<const bf16x8_t*>(qrow + c * 32) : zero;
+  }
+  [[maybe_unused]] float gain[FRESH ? DC * 8 : 1];
+  [[maybe_unused]] float4 angle[FRESH ? HC * 4 : 1];  // (cos, sin) of two pairs each
+  [[maybe_unused]] bool fresh_here = false;           // this workgroup's keys include the token's own
+  [[maybe_unused]] int slot = -1;
+  [[maybe_unused]] bf16 ka[PAIRS], kb2[PAIRS], vv[2 * PAIRS];
+  [[maybe_unused]] float gka[PAIRS], gkb[PAIRS];
+  [[maybe_unused]] float2 kcs[PAIRS];
+  if constexpr (FRESH != 0) {
+#pragma unroll
+    for (int c = 0; c < HC; ++c) {
+      const int i0 = c * 32 + grp * 8;
+      load_gains8((const W*)fresh.qw + i0, &gain[c * 8]);
+      load_gains8((const W*)fresh.qw + i0 + HALF, &gain[(c + HC) * 8]);
+      const float4* cs4 = reinterpret_cast<const float4*>(fresh.cs + (size_t)t * HALF + i0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) angle[c * 4 + j] = cs4[j];
+    }
+    fresh_here = fresh.store && pos >= k0 && pos < k1;  // the same for the whole workgroup
+    if (fresh_here && wave == 0) {
+      slot = fresh.slots[t];
+      const bf16* src = fresh.qkv + (row + H + kvh) * D;
+#pragma unroll
+      for (int p = 0; p < PAIRS; ++p) {
+        const int i = min(lane + p * WAVE, HALF - 1);
+        ka[p] = src[i];
+        kb2[p] = src[i + HALF];
+        gka[p] = (float)((const W*)fresh.kw)[i];
+        gkb[p] = (float)((const W*)fresh.kw)[i + HALF];
+        kcs[p] = fresh.cs[(size_t)t * HALF + i];
+      }
+    } else if (fresh_here && wave == 1) {
+      slot = fresh.slots[t];
+      const bf16* src = fresh.qkv + (row + H + KV + kvh) * D;
+#pragma unroll
+      for (int p = 0; p < 2 * PAIRS; ++p) vv[p] = src[min(lane + p * WAVE, D - 1)];
+    }
+  }
+  const int first = (k0 / 32) * 32;
+  KVStep<DC> cur, nxt;
+  int kb = first + 32 * wave;
+  if (kb < k1) load_kv_step<DC>(cur, k_pages, v_pages, table, kb, k1, KV, kvh, bs, col, grp);
+
+  if constexpr (FRESH != 0) {
+    // the queries of this lane's head: norm over the head (its D values lie in four lanes), rotation
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += (float)qop[c][j] * (float)qop[c][j];
+    ss += __shfl_xor(ss, 16, WAVE);
+    ss += __shfl_xor(ss, 32, WAVE);
+    const float inv = 1.0f / sqrtf(ss / (float)D + fresh.eps);
+#pragma unroll
+    for (int c = 0; c < HC; ++c)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float a = (float)qop[c][j] * inv * gain[c * 8 + j];
+        const float b = (float)qop[c + HC][j] * inv * gain[(c + HC) * 8 + j];
+        const float4 cs2 = angle[c * 4 + j / 2];
+        const float cc = (j & 1) ? cs2.z : cs2.x, sn = (j & 1) ? cs2.w : cs2.y;
+        qop[c][j] = (bf16)(a * cc - b * sn);
+        qop[c + HC][j] = (bf16)(b * cc + a * sn);
+      }
+    if (col >= G) {
+#pragma unroll
+      for (int c = 0; c < DC; ++c) qop[c] = zero;
+    }
+    if (fresh_here) {
+      const size_t head = slot >= 0 ? ((size_t)(slot / bs) * KV + kvh) * bs * D : 0;
+      if (wave == 0) {  // the key: norm and rotation as for the queries, one wave over the pairs
+        float ks = 0.f;
+#pragma unroll
+        for (int p = 0; p < PAIRS; ++p)
+          if (lane + p * WAVE < HALF) ks += (float)ka[p] * (float)ka[p] + (float)kb2[p] * (float)kb2[p];
+        ks = wave_sum(ks);
+        const float kinv = 1.0f / sqrtf(ks / (float)D + fresh.eps);
+        bf16* dst = fresh.k_store + head + (size_t)(slot % bs) * D;
+#pragma unroll
+        for (int p = 0; p < PAIRS; ++p) {
+          const int i = lane + p * WAVE;
+          if (i < HALF) {
+            const float a = (float)ka[p] * kinv * gka[p], b = (float)kb2[p] * kinv * gkb[p];
+            const bf16 ra = (bf16)(a * kcs[p].x - b * kcs[p].y), rb = (bf16)(b * kcs[p].x + a * kcs[p].y);
+            fresh_kv[0][i] = ra;
+            fresh_kv[0][i + HALF] = rb;
+            if (slot >= 0) { dst[i] = ra; dst[i + HALF] = rb; }
+          }
+        }
+      } else if (wave == 1) {  // the value, as it is; its page is stored transposed
+        bf16* vt = fresh.v_store + head + slot % bs;
+#pragma unroll
+        for (int p = 0; p < 2 * PAIRS; ++p) {
+          const int i = lane + p * WAVE;
+          if (i < D) {
+            fresh_kv[1][i] = vv[p];
+            if (slot >= 0) vt[(size_t)i * bs] = vv[p];
+          }
+        }
+      }
+      __syncthreads();
+    }
   }
   f32x4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = NEG_INF, l = 0.f;
 
-  const int first = (k0 / 32) * 32;
-  KVStep<DC> cur, nxt;
-  int kb = first + 32 * wave;
-  if (kb < k1) load_kv_step<DC>(cur, k_pages, v_pages, table, kb, k1, KV, kvh, bs, col, grp);
   for (; kb < k1; kb += 128) {
     const bool more = kb + 128 < k1;
     if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 128, k1, KV, kvh, bs, col, grp);
+    if constexpr (FRESH != 0) {
+      if (fresh_here && pos >= kb && pos < kb + 32) {  // this wave's step holds the token itself: take it from LDS
+        const int at = pos - kb;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          if ((at >> 4) != tt) continue;
+          if (col == (at & 15)) {
+#pragma unroll
+            for (int c = 0; c < DC; ++c) cur.k[tt][c] = *reinterpret_cast<const bf16x8_t*>(&fresh_kv[0][c * 32 + grp * 8]);
+          }
+          if (grp == ((at & 15) >> 2)) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                if (r == (at & 3)) cur.v[tt][dt][r] = fresh_kv[1][dt * 16 + col];
+          }
+        }
+      }
+    }
     // ---- scores of 32 keys
     f32x4_t s[2];
 #pragma unroll
@@ -775,25 +931,42 @@ static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_
                               int num_items, const int* positions, const int* tok_row, const int* block_tables,
                               int table_width, void* out, float* part_m, float* part_l, float* part_acc, int H,
                               int KV, int D, int bs, float scale, int window, int part_size, int P,
-                              hipStream_t stream) {
+                              const FreshQKV* fresh, int gains_dtype, hipStream_t stream) {
   const int G = H / KV;
   if (D % 32 || D > 256 || G > 16 || bs % 16 || part_size % 32) return AS_BAD_SHAPE;
+  if (fresh && D % 64) return AS_BAD_SHAPE;
   dim3 grid(num_items, KV, P);
   const size_t shmem = sizeof(float) * (size_t)(128 + 4 * D * G);
-#define LAUNCH(DCV)                                                                                       \
-  attn_decode_mfma_kernel<DCV><<<grid, 256, shmem, stream>>>(                                             \
+  const FreshQKV none = {};
+#define LAUNCH(DCV, FRESHV)                                                                               \
+  attn_decode_mfma_kernel<DCV, FRESHV><<<grid, 256, shmem, stream>>>(                                     \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, items, positions, tok_row, block_tables, \
-      table_width, (bf16*)out, part_m, part_l, part_acc, H, KV, bs, scale, window, part_size, P)
-  switch (D / 32) {
-    case 1: LAUNCH(1); break;
-    case 2: LAUNCH(2); break;
-    case 3: LAUNCH(3); break;
-    case 4: LAUNCH(4); break;
-    case 5: LAUNCH(5); break;
-    case 6: LAUNCH(6); break;
-    case 7: LAUNCH(7); break;
-    default: LAUNCH(8); break;
+      table_width, (bf16*)out, part_m, part_l, part_acc, H, KV, bs, scale, window, part_size, P,          \
+      FRESHV ? *fresh : none)
+#define LAUNCH_FRESH(FRESHV)            \
+  switch (D / 64) {                     \
+    case 1: LAUNCH(2, FRESHV); break;   \
+    case 2: LAUNCH(4, FRESHV); break;   \
+    case 3: LAUNCH(6, FRESHV); break;   \
+    default: LAUNCH(8, FRESHV); break;  \
   }
+  if (fresh && gains_dtype == DT_F32) {
+    LAUNCH_FRESH(2)
+  } else if (fresh) {
+    LAUNCH_FRESH(1)
+  } else {
+    switch (D / 32) {
+      case 1: LAUNCH(1, 0); break;
+      case 2: LAUNCH(2, 0); break;
+      case 3: LAUNCH(3, 0); break;
+      case 4: LAUNCH(4, 0); break;
+      case 5: LAUNCH(5, 0); break;
+      case 6: LAUNCH(6, 0); break;
+      case 7: LAUNCH(7, 0); break;
+      default: LAUNCH(8, 0); break;
+    }
+  }
+#undef LAUNCH_FRESH
 #undef LAUNCH
   if (hipGetLastError() != hipSuccess) return AS_LAUNCH_FAILED;
   if (P > 1) {
@@ -814,7 +987,31 @@ extern "C" int as_attn_decode_mfma(const void* q, const void* k_pages, const voi
     return AS_BAD_SHAPE;
   if (P > 1 && (!part_m || !part_l || !part_acc)) return AS_BAD_SHAPE;
   return launch_decode_mfma(q, k_pages, v_pages, items, num_items, positions, tok_row, block_tables, table_width,
-                            out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size, P, stream);
+                            out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size, P, nullptr,
+                            DT_BF16, stream);
+}
+
+// A decode step (token t is row t of the block tables) from the projection's output: per-head norm,
+// rotation of the whole head, the new token's key and value written to its slot (store 0: queries
+// only, the pages already hold them), and attention, in one kernel.  qkv [T, H + 2 KV, D] bf16;
+// qw, kw [D] bf16 or fp32; cs [T, D/2] float2; slots [T].  Needs D % 64 == 0.
+extern "C" int as_attn_decode_fresh(const void* qkv, const void* qw, const void* kw, int gains_dtype,
+                                    const float* cs, const int* slots, float eps, int store, void* k_pages,
+                                    void* v_pages, int num_tokens, const int* positions,
+                                    const int* block_tables, int table_width, void* out, float* part_m,
+                                    float* part_l, float* part_acc, int H, int KV, int D, int bs, float scale,
+                                    int window, int part_size, int P, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || H % KV || D <= 0 || bs <= 0 || part_size <= 0 || P <= 0 || table_width <= 0)
+    return AS_BAD_SHAPE;
+  if (P > 1 && (!part_m || !part_l || !part_acc)) return AS_BAD_SHAPE;
+  if (!qkv || !qw || !kw || !cs || (store && !slots)) return AS_BAD_SHAPE;
+  if (gains_dtype != DT_BF16 && gains_dtype != DT_F32) return AS_BAD_DTYPE;
+  const FreshQKV fresh = {(const bf16*)qkv, qw, kw, (const float2*)cs, slots, (bf16*)k_pages, (bf16*)v_pages,
+                          eps, store};
+  return launch_decode_mfma(nullptr, k_pages, v_pages, nullptr, num_tokens, positions, nullptr, block_tables,
+                            table_width, out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size,
+                            P, &fresh, gains_dtype, stream);
 }
 
 static int pow2ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }

@@ -163,9 +163,27 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
                           f"(needs a multiple of {chunk}, at most {SINGLE_QUERY_MAX_HEAD_DIM})")  # fmt: skip
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
-    span = min(max_context, window) if window > 0 else max_context
     G = H // KV
     mfma = q.dtype == BF16 and D % 32 == 0 and G <= 16 and bs % 16 == 0 and not force_generic
+    part_size, P, part_m, part_l, part_acc = _partitions(N, H, KV, D, max_context, window, mfma, part_size, q.device)
+    if mfma:
+        call("as_attn_decode_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, _ptr(positions),
+             _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
+             _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+        return
+    call("as_attn_single_query", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(items), N,
+         _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m),
+         _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+
+
+ATTN_FILL_GROUPS = 512  # (token, kv head) pairs that occupy every compute unit twice over
+
+
+def _partitions(N, H, KV, D, max_context, window, mfma, part_size, device):
+    """How the keys of N single queries are cut for the split-KV kernels, and the buffers of the
+    partial results: (part_size, P, part_m, part_l, part_acc), the buffers None when P == 1."""
+    span = min(max_context, window) if window > 0 else max_context
+    G = H // KV
     if part_size is None:
         # Enough partitions to occupy the GPU when few tokens are in the batch, few enough that
         # the merge stays small; boundaries are multiples of part_size in absolute position.
@@ -184,20 +202,60 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
     P = max(1, math.ceil(max_context / part_size))
     part_m = part_l = part_acc = None
     if P > 1:
-        part_m = torch.empty((N, H, P), dtype=F32, device=q.device)
-        part_l = torch.empty((N, H, P), dtype=F32, device=q.device)
-        part_acc = torch.empty((N, H, P, D), dtype=F32, device=q.device)
-    if mfma:
-        call("as_attn_decode_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, _ptr(positions),
-             _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
-             _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+        part_m = torch.empty((N, H, P), dtype=F32, device=device)
+        part_l = torch.empty((N, H, P), dtype=F32, device=device)
+        part_acc = torch.empty((N, H, P, D), dtype=F32, device=device)
+    return part_size, P, part_m, part_l, part_acc
+
+
+def attn_decode_fresh_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, block_size: int,
+                                rotary_dim: int, qk_norm: bool) -> bool:
+    """Whether `attn_decode_fresh` takes this case: bfloat16 heads of 64, 128, 192 or 256 with a per-head
+    norm, rotated whole, at most 16 query heads to a kv head, pages of a multiple of 16 tokens."""
+    return (dtype == BF16 and head_dim % 64 == 0 and head_dim <= 256 and rotary_dim == head_dim and qk_norm
+            and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16 and block_size % 16 == 0)  # fmt: skip
+
+
+def attn_decode_fresh(qkv, q_weight, k_weight, cos_sin, slots, eps, store_kv, k_pages, v_pages, positions,
+                      block_tables, out, num_heads, scale, window, max_context, part_size=None) -> None:
+    """A decode step from the projection's output, in one kernel: what `qk_norm_rope_store` and then
+    `attn_single_query` do for tokens that are their own rows (token t reads block table t).
+
+    qkv [T, H + 2 KV, D] bf16; q_weight, k_weight [D] bf16 or fp32; cos_sin [T, D/2, 2] fp32;
+    slots [T] int32; store_kv False: queries only, the pages already hold the tokens' keys and values
+    (a run that reads another run's cache); out [T, H, D]."""
+    _check(qkv, "qkv", BF16, (None, None, None))
+    T, heads, D = qkv.shape
+    H = num_heads
+    _check(k_pages, "k_pages", BF16, (None, None, None, D))
+    _, KV, bs, _ = k_pages.shape
+    if heads != H + 2 * KV:
+        raise KernelError(f"qkv has {heads} heads, expected {H} + 2 x {KV}")
+    _check(v_pages, "v_pages", BF16, (k_pages.shape[0], KV, D, bs))
+    _check(out, "out", BF16, (T, H, D))
+    _check(positions, "positions", I32, (T,))
+    _check(block_tables, "block_tables", I32, (None, None))
+    if block_tables.shape[0] < T:
+        raise KernelError(f"attention: {T} tokens that are their own rows need as many block tables")
+    R = 2 * cos_sin.shape[1] if cos_sin is not None else 0
+    if not attn_decode_fresh_supported(BF16, H, KV, D, bs, R, q_weight is not None and k_weight is not None):
+        raise KernelError(f"attention from fresh projections: unsupported heads {H}/{KV}, head width {D}, "
+                          f"rotary width {R}, page size {bs}, or no per-head norm")  # fmt: skip
+    _check(cos_sin, "cos_sin", F32, (T, D // 2, 2))
+    _check(q_weight, "q_weight", (F32, BF16), (D,))
+    _check(k_weight, "k_weight", q_weight.dtype, (D,))
+    w_dtype = q_weight.dtype
+    if store_kv:
+        _check(slots, "slots", I32, (T,))
+    if T == 0:
         return
-    call("as_attn_single_query", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(items), N,
-         _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m),
-         _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
-
-
-ATTN_FILL_GROUPS = 512  # (token, kv head) pairs that occupy every compute unit twice over
+    if max_context > block_tables.shape[1] * bs:
+        raise KernelError("attention: block tables are shorter than the longest context")
+    part_size, P, part_m, part_l, part_acc = _partitions(T, H, KV, D, max_context, window, True, part_size, qkv.device)
+    call("as_attn_decode_fresh", _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _DT[w_dtype], _ptr(cos_sin),
+         _ptr(slots) if store_kv else 0, float(eps), int(bool(store_kv)), _ptr(k_pages), _ptr(v_pages), T,
+         _ptr(positions), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
+         _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 PREFILL_MAX_HEAD_DIM = 256  # four stages of 32 keys and values of such heads fill 128 KB of LDS
 
 

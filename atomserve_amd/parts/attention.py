@@ -69,15 +69,26 @@ class Attention(Mixer):
             h.gemm(self.qkv_weight, qkv)
         else:
             ops.gemm(h, self.qkv_weight, qkv)
-        q = torch.empty((T, H, D), dtype=env.dtype, device=device)
         cos_sin = self.position.prepare(step) if self.position is not None else None
         eps = s.qk_norm.eps if s.qk_norm is not None else 0.0
-        ops.qk_norm_rope_store(
-            qkv.view(T, H + 2 * KV, D), self.q_norm_weight, self.k_norm_weight, cos_sin, cache.slots, q,
-            cache.k_pages, cache.v_pages, H, KV, eps, store_kv=cache.writes,
-        )  # fmt: skip
-        out = torch.empty((T, H, D), dtype=env.dtype, device=device)
-        self.attend(q, out, step, cache)
+        rotary = 2 * cos_sin.shape[1] if cos_sin is not None else 0
+        if step.decode_only and ops.attn_decode_fresh_supported(env.dtype, H, KV, D, cache.block_size, rotary,
+                                                                s.qk_norm is not None):  # fmt: skip
+            # a decode step: norm, rotation, the cache store and attention in one kernel
+            out = torch.empty((T, H, D), dtype=env.dtype, device=device)
+            ops.attn_decode_fresh(
+                qkv.view(T, H + 2 * KV, D), self.q_norm_weight, self.k_norm_weight, cos_sin, cache.slots, eps,
+                cache.writes, cache.k_pages, cache.v_pages, step.positions, cache.block_tables, out, H, s.scale,
+                s.window, step.max_context,
+            )  # fmt: skip
+        else:
+            q = torch.empty((T, H, D), dtype=env.dtype, device=device)
+            ops.qk_norm_rope_store(
+                qkv.view(T, H + 2 * KV, D), self.q_norm_weight, self.k_norm_weight, cos_sin, cache.slots, q,
+                cache.k_pages, cache.v_pages, H, KV, eps, store_kv=cache.writes,
+            )  # fmt: skip
+            out = torch.empty((T, H, D), dtype=env.dtype, device=device)
+            self.attend(q, out, step, cache)
         if residual is not None and next_norm is not None:
             link = next_norm.absorb(out.view(T, H * D), self.o_weight, residual)
             if link is not None:

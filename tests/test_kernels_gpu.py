@@ -526,6 +526,71 @@ def test_attention_of_a_decode_step_needs_no_maps(ops, dtype):
         ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables[:3], b, D**-0.5, 0, max(lens))
 
 
+@pytest.mark.parametrize("H,KV,D,bs,gain,window", [
+    (32, 8, 128, 16, BF16, 0), (6, 2, 64, 32, F32, 0), (14, 2, 192, 16, BF16, 40), (5, 5, 256, 16, BF16, 0),
+    (16, 1, 128, 48, F32, 0), (8, 2, 128, 16, BF16, 1),
+])  # fmt: skip
+@pytest.mark.parametrize("part", [None, 32, 128])
+def test_decode_step_from_fresh_projections(ops, H, KV, D, bs, gain, window, part):
+    """Norm, rotation, cache store and attention of a decode step in one kernel: against the plain
+    functions, and against the two kernels it stands for.  Contexts end at the first and the last
+    slot of a page, at the edges of the partitions and of a wave's 32 keys; one row keeps its token
+    out of the pages (slot -1) and still attends it; with `store_kv` off nothing is written and the
+    key that the pages hold is attended."""
+    lens = [1, 16, 17, 32, 33, 128, 129, 300, 512, 513, 1000]
+    _, k_pages, v_pages, tables, positions = paged_case(BF16, H, KV, D, bs, lens, seed=5, k_scale=3.0 / math.sqrt(D / 16))
+    T = len(lens)
+    g = torch.Generator().manual_seed(9)
+    qkv = (torch.randn(T, H + 2 * KV, D, generator=g) * 2).to(BF16).to(DEV)
+    qw, kw = (torch.randn(D, generator=g) + 1).to(gain).to(DEV), (torch.randn(D, generator=g) + 1).to(gain).to(DEV)
+    inv = (1.0 / (1e4 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))).to(DEV)
+    cs = torch.empty(T, D // 2, 2, device=DEV)
+    ops.rope_table(positions, inv, cs)
+    slot_list = [tables[i, (n - 1) // bs].item() * bs + (n - 1) % bs for i, n in enumerate(lens)]
+    slot_list[3] = -1  # this row's token stays out of the pages
+    slots = i32(slot_list)
+    scale = D**-0.5
+    rows = i32(list(range(T)))
+    # plain: the new keys and values go to the pages, then every query attends its context
+    rq, rk, rv = pk.qk_norm_rope(qkv, qw, kw, cs, H, KV, 1e-6)
+    ref_k, ref_v = k_pages.float(), v_pages.float()
+    pk.store_pages(ref_k, ref_v, rk, rv, i32([tables[i, (n - 1) // bs].item() * bs + (n - 1) % bs for i, n in enumerate(lens)]))
+    ref = pk.paged_attention(rq.to(BF16), ref_k.to(BF16), ref_v.to(BF16), rows, positions, rows, tables, scale, window)
+    # the two kernels
+    k2, v2 = k_pages.clone(), v_pages.clone()
+    q2, out2 = torch.empty(T, H, D, dtype=BF16, device=DEV), torch.zeros(T, H, D, dtype=BF16, device=DEV)
+    ops.qk_norm_rope_store(qkv, qw, kw, cs, slots, q2, k2, v2, H, KV, 1e-6)
+    ops.attn_single_query(q2, k2, v2, None, positions, None, tables, out2, scale, window, max(lens), part)
+    # the one kernel
+    k1, v1 = k_pages.clone(), v_pages.clone()
+    out1 = torch.zeros(T, H, D, dtype=BF16, device=DEV)
+    ops.attn_decode_fresh(qkv, qw, kw, cs, slots, 1e-6, True, k1, v1, positions, tables, out1, H, scale, window, max(lens), part)
+    torch.cuda.synchronize()
+    assert torch.equal(v1, v2)
+    assert close_bf16(k1, k2.float()) and (k1 != k2).float().mean() < 0.02  # the squares are summed in another order
+    written = torch.zeros(k_pages.shape[0] * bs, dtype=torch.bool, device=DEV)
+    written[slots[slots >= 0].long()] = True
+    untouched = ~written.view(-1, bs)  # [page, offset]: nothing but the slots was written
+    assert torch.equal(k1.permute(0, 2, 1, 3)[untouched], k_pages.permute(0, 2, 1, 3)[untouched])
+    assert torch.equal(v1.permute(0, 3, 1, 2)[untouched], v_pages.permute(0, 3, 1, 2)[untouched])
+    assert torch.allclose(out1.float(), ref, atol=2e-2, rtol=2e-2)
+    keep = [i for i in range(T) if i != 3]  # the two kernels cannot attend a token that they keep out of the pages
+    assert torch.allclose(out1[keep].float(), out2[keep].float(), atol=2e-2, rtol=2e-2)
+    # queries only: the pages as the plain store left them are read, nothing is written
+    k3, v3 = ref_k.to(BF16), ref_v.to(BF16)
+    before_k, before_v = k3.clone(), v3.clone()
+    out3 = torch.zeros(T, H, D, dtype=BF16, device=DEV)
+    ops.attn_decode_fresh(qkv, qw, kw, cs, None, 1e-6, False, k3, v3, positions, tables, out3, H, scale, window, max(lens), part)
+    torch.cuda.synchronize()
+    assert torch.equal(k3, before_k) and torch.equal(v3, before_v)
+    assert torch.allclose(out3.float(), ref, atol=2e-2, rtol=2e-2)
+    # heads without a norm or a whole rotation are left to the two kernels
+    for weights, angles in ((None, cs), (qw, None), (qw, cs[:, : D // 4].contiguous())):
+        with pytest.raises(ops.KernelError, match="fresh projections"):
+            ops.attn_decode_fresh(qkv, weights, weights, angles, slots, 1e-6, True, k3, v3, positions, tables, out3, H,
+                                  scale, window, max(lens), part)  # fmt: skip
+
+
 def test_attention_of_a_batch_that_fills_the_gpu(ops):
     """64 requests of 8 kv heads are 512 workgroups already: the contexts are not partitioned (no
     merge), each workgroup walks its whole context, of very different lengths."""
