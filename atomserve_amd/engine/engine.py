@@ -6,6 +6,10 @@
     scheduler.update(plan, results)
     push each new token to its request's handle
 
+While nothing changes among the running requests (all decode, nobody waits, nobody reaches its
+length), the next decode step goes to the GPU before this one's tokens are read: the GPU passes
+the sampled tokens on by itself, and the host's share of a step is hidden behind the GPU's.
+
 Clients on any thread talk to it through queues only: one inbox for submit and abort,
 one outbox per request that streams its tokens back.  It deals in token ids only.
 """
@@ -23,7 +27,7 @@ from typing import Optional
 from atomserve_amd.cache.manager import CacheManager
 from atomserve_amd.config.engine_config import EngineConfig
 from atomserve_amd.engine.runner import ModelRunner
-from atomserve_amd.engine.scheduler import Scheduler
+from atomserve_amd.engine.scheduler import Scheduler, SchedulerOutput
 from atomserve_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus
 from atomserve_amd.kernels import ops
 
@@ -85,6 +89,8 @@ class Engine:
         self._thread: Optional[threading.Thread] = None
         self._stopping = False
         self._rng = random.Random(seed)  # seeds of the requests that bring none
+        self._in_flight = None  # (plan, pending step) of a decode step sent to the GPU ahead of its turn
+        self.run_ahead = True
         self.num_steps = 0
         self.last_batch_seqs = 0
         self.last_batch_tokens = 0
@@ -165,12 +171,24 @@ class Engine:
     def step(self) -> bool:
         """One scheduling step; False when there is nothing to do."""
         self._drain_inbox(block=False)
-        if not self.scheduler.has_work:
-            return False
-        out = self.scheduler.schedule()
-        if not out.seqs:
-            raise RuntimeError("scheduler has work but scheduled nothing")
-        results = self.runner.execute(out)
+        flight, self._in_flight = self._in_flight, None
+        if flight is not None:
+            out, pending = flight  # planned and sent to the GPU during the step before
+        else:
+            if not self.scheduler.has_work:
+                return False
+            out = self.scheduler.schedule()
+            if not out.seqs:
+                raise RuntimeError("scheduler has work but scheduled nothing")
+            launch = getattr(self.runner, "launch", None)
+            pending = launch(out) if launch is not None else None
+        if pending is None:
+            results = self.runner.execute(out)
+        else:
+            ahead = self._plan_ahead(out)
+            if ahead is not None:
+                self._in_flight = (ahead, self.runner.launch(ahead, after=pending))
+            results = pending.results()
         new_tokens = self.scheduler.update(out, results)
 
         now = time.perf_counter()
@@ -188,6 +206,32 @@ class Engine:
             if seq.status is SequenceStatus.FINISHED:
                 self._close(seq)
         return True
+
+    def _plan_ahead(self, out):
+        """The decode step after `out`, if it is certain but for its tokens: `out` gives every running
+        request a token, nobody waits or has left, nobody reaches its length with that token, no sampling
+        setting needs the tokens on the host, and every request has a page for one more position.  A
+        request that ends on an end-of-sequence token in `out` still takes part in the step ahead; its
+        result there is dropped and its pages, given back at once, may be written once more, which is
+        harmless: whoever gets them next writes after that, in the order of the GPU's queue."""
+        s = self.scheduler
+        can = getattr(self.runner, "can_run_ahead", None)
+        if not self.run_ahead or can is None or out.preempted or s.waiting or not self._inbox.empty():
+            return None
+        if len(out.seqs) != len(s.running) or any(a is not b for a, b in zip(out.seqs, s.running)):
+            return None
+        limit = s.config.max_model_len
+        for seq, n in zip(out.seqs, out.num_new_tokens):
+            p = seq.params
+            if (seq.status is not SequenceStatus.RUNNING or not seq.reaches_end(n) or p.presence_penalty != 0
+                    or seq.num_output_tokens + 1 >= p.max_tokens or seq.num_tokens + 1 >= limit):  # fmt: skip
+                return None
+        if not can(out.seqs):
+            return None
+        for seq in out.seqs:
+            if not s.manager.reserve(seq.cache, seq.num_tokens, 1):
+                return None  # the scheduler decides who makes room, in its own turn
+        return SchedulerOutput(seqs=list(out.seqs), num_new_tokens=[1] * len(out.seqs))
 
     def _drain_inbox(self, block: bool) -> None:
         while True:
@@ -221,6 +265,7 @@ class Engine:
                     self._drain_inbox(block=True)
             except Exception as error:  # fail the requests, keep the engine alive
                 traceback.print_exc(file=sys.stderr)
+                self._in_flight = None
                 for seq in [*self.scheduler.running, *self.scheduler.waiting]:
                     self.scheduler.abort(seq.id)
                     seq.finish_reason = "error"

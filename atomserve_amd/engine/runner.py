@@ -74,7 +74,9 @@ class DecodeGraphs:
             and all(len(row.tokens) == 1 for row in rows)
         )
 
-    def run(self, rows):
+    def run(self, rows, tokens_from=None):
+        """tokens_from: int32 [len(rows)] on the GPU, the rows' tokens where the host does not know them
+        yet (the step before is still running); copied into the step's buffer after the host's integers."""
         r = self.runner
         bs = r.manager.block_size
         n = _bucket(len(rows), self.ROW_BUCKETS)
@@ -92,6 +94,8 @@ class DecodeGraphs:
             while len(self.graphs) >= self.MAX_GRAPHS:
                 self.graphs.popitem(last=False)
             batch = r.prepare(padded, table_width=width, max_context=context)
+            if tokens_from is not None:
+                batch.token_ids[: len(rows)].copy_(tokens_from)
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -120,10 +124,13 @@ class DecodeGraphs:
                 if collecting:
                     gc.enable()
             entry = self.graphs[key] = (graph, batch, logits)
-        elif not entry[1].advance(padded):
-            # other requests than last time, or a window moved: pack anew into the captured buffer
-            batch = r.prepare(padded, table_width=width, max_context=context, into=entry[1])
-            entry = self.graphs[key] = (entry[0], batch, entry[2])
+        else:
+            if not entry[1].advance(padded):
+                # other requests than last time, or a window moved: pack anew into the captured buffer
+                batch = r.prepare(padded, table_width=width, max_context=context, into=entry[1])
+                entry = self.graphs[key] = (entry[0], batch, entry[2])
+            if tokens_from is not None:
+                entry[1].token_ids[: len(rows)].copy_(tokens_from)
         graph, batch, logits = entry
         graph.replay()
         wanted = [i for i, row in enumerate(rows) if row.want]
@@ -147,6 +154,29 @@ class DecodeGraphs:
         return len(self.graphs) - before
 
 
+class _Passed:
+    def synchronize(self) -> None:
+        pass
+
+
+class PendingStep:
+    """A step that is on the GPU, sampling included; `results()` waits for its tokens."""
+
+    def __init__(self, samples, num_computed, device_tokens, host_tokens, event):
+        self.samples = samples  # per scheduled sequence: whether the step gives it a token
+        self.num_computed = num_computed  # per scheduled sequence: its leading tokens in the cache afterwards
+        self.device_tokens = device_tokens  # int32 on the GPU, one per sampling sequence, or None
+        self.host_tokens = host_tokens  # pinned; filled when `event` has passed
+        self.event = event
+
+    def results(self) -> list:
+        tokens = iter(())
+        if self.device_tokens is not None:
+            self.event.synchronize()
+            tokens = iter(self.host_tokens[: self.device_tokens.shape[0]].tolist())
+        return [StepResult([next(tokens)] if yes else [], n) for yes, n in zip(self.samples, self.num_computed)]
+
+
 class ModelRunner:
     """Owns the model, the cache pools and the sampler; executes one step for a list of rows."""
 
@@ -159,18 +189,23 @@ class ModelRunner:
         self.staging = Staging(self.device)
         self.vocab_size = model.plan.vocab_size
         self.decode_graphs = DecodeGraphs(self) if use_graphs else None
+        self._token_buffers = []  # pinned, used in turn: the sampled tokens of the steps on their way
+        self._token_turn = 0
 
     def prepare(self, rows, **layout) -> StepBatch:
         return StepBatch(rows, self.manager.block_size, len(self.manager.paged_groups), self.vocab_size,
                          self.device, pools=self.pools, staging=self.staging, **layout)  # fmt: skip
 
     @torch.inference_mode()
-    def step(self, rows) -> torch.Tensor:
-        """Logits [sum of len(row.want), vocab] fp32, in the order of the rows and of `want`."""
+    def step(self, rows, tokens_from=None) -> torch.Tensor:
+        """Logits [sum of len(row.want), vocab] fp32, in the order of the rows and of `want`.
+        tokens_from: see `DecodeGraphs.run`; for decode steps that are replayed only."""
         if self.decode_graphs is not None and self.decode_graphs.eligible(rows):
             if any(w != 0 for row in rows for w in row.want):
                 raise ValueError("a row wants logits at a place outside its tokens")
-            return self.decode_graphs.run(rows)
+            return self.decode_graphs.run(rows, tokens_from)
+        if tokens_from is not None:
+            raise ValueError("only a replayed decode step takes its tokens from the GPU")
         batch = self.prepare(rows)
         return self.model.forward(batch)
 
@@ -180,14 +215,48 @@ class ModelRunner:
         reaches its end this step (reference atomserve/runner.py:182-192)."""
         return self.step(rows_for(seqs, num_new_tokens))
 
-    @torch.inference_mode()
     def execute(self, out) -> list:
         """Run one scheduled step and sample: a sequence that reaches the end of its known
         tokens gets one new token (reference atomserve/runner.py:194-212)."""
-        logits = self.step(rows_for(out.seqs, out.num_new_tokens))
-        sampling = [s for s, n in zip(out.seqs, out.num_new_tokens, strict=True) if s.reaches_end(n)]
-        sampled = iter(self.sampler.sample(logits, sampling))
-        return [
-            StepResult(tokens=[next(sampled)] if seq.reaches_end(n) else [], num_computed=seq.num_computed_tokens + n)
-            for seq, n in zip(out.seqs, out.num_new_tokens, strict=True)
-        ]
+        return self.launch(out).results()
+
+    def can_run_ahead(self, seqs) -> bool:
+        """Whether a decode step of these sequences can go to the GPU before the step before it has been
+        read: it must be a replayed step, whose token buffer the GPU can fill itself."""
+        graphs = self.decode_graphs
+        return graphs is not None and graphs.eligible([Row([0], 0, graphs.filler_tables, [0], -1)] * len(seqs))
+
+    @torch.inference_mode()
+    def launch(self, out, after: PendingStep = None) -> PendingStep:
+        """Put one scheduled step on the GPU, sampling included, without waiting for it.
+
+        after: the step before it, not read yet, when this one runs ahead.  Then every sequence decodes
+        the token that `after` samples for it, which the GPU hands over itself, at the position after its
+        last known token; the sequences' own bookkeeping is one step behind until `after` is read."""
+        if after is None:
+            samples = [s.reaches_end(n) for s, n in zip(out.seqs, out.num_new_tokens, strict=True)]
+            num_computed = [s.num_computed_tokens + n for s, n in zip(out.seqs, out.num_new_tokens)]
+            logits = self.step(rows_for(out.seqs, out.num_new_tokens))
+        else:
+            samples = [True] * len(out.seqs)
+            num_computed = [s.num_tokens + 1 for s in out.seqs]
+            rows = [Row([0], s.num_tokens, s.cache.tables, [0], s.cache.state_slot) for s in out.seqs]
+            logits = self.step(rows, tokens_from=after.device_tokens)
+        sampling = [s for s, yes in zip(out.seqs, samples) if yes]
+        device_tokens = self.sampler.launch(logits, sampling, ahead=0 if after is None else 1)
+        host_tokens = event = None
+        if device_tokens is not None:
+            if device_tokens.is_cuda:
+                if len(self._token_buffers) < 3:
+                    self._token_buffers.append(torch.empty(4096, dtype=torch.int32, pin_memory=True))
+                self._token_turn = (self._token_turn + 1) % len(self._token_buffers)
+                host_tokens = self._token_buffers[self._token_turn]
+                if host_tokens.numel() < device_tokens.shape[0]:
+                    host_tokens = self._token_buffers[self._token_turn] = torch.empty(
+                        device_tokens.shape[0], dtype=torch.int32, pin_memory=True)  # fmt: skip
+                host_tokens[: device_tokens.shape[0]].copy_(device_tokens, non_blocking=True)
+                event = torch.cuda.Event()
+                event.record()
+            else:
+                host_tokens, event = device_tokens, _Passed()
+        return PendingStep(samples, num_computed, device_tokens, host_tokens, event)

@@ -116,6 +116,8 @@ class Scheduler:
         (sequence, its new tokens) for every sequence that got any."""
         new_tokens = []
         for seq, result in zip(out.seqs, results, strict=True):
+            if seq.status is not SequenceStatus.RUNNING:
+                continue  # finished or aborted while the step was on its way: its result is dropped
             appended = []
             for token in result.tokens:
                 seq.token_ids.append(token)

@@ -27,8 +27,15 @@ class Sampler:
     def sample(self, logits: torch.Tensor, seqs) -> list:
         """logits [B, vocab] fp32, row i belongs to seqs[i]; returns B token ids (one host
         synchronisation, the step's only one)."""
+        out = self.launch(logits, seqs)
+        return [] if out is None else out.tolist()
+
+    def launch(self, logits: torch.Tensor, seqs, ahead: int = 0):
+        """The same without waiting: the B token ids as an int32 tensor on the GPU (None for no rows).
+        ahead: how many tokens each sequence will have sampled by then beyond what it holds now (a step
+        put on the GPU before the one before it was read)."""
         if not seqs:
-            return []
+            return None
         B, vocab = logits.shape
         if B != len(seqs):
             raise ValueError(f"{B} rows of logits for {len(seqs)} sequences")
@@ -37,7 +44,7 @@ class Sampler:
         out = torch.empty(B, dtype=torch.int32, device=self.device)
         if all(p.temperature == 0 for p in params):
             ops.argmax(logits, out)
-            return out.tolist()
+            return out
         top_k, kept = [], []
         for p in params:
             k = p.top_k if 0 < p.top_k < vocab else 0
@@ -51,13 +58,13 @@ class Sampler:
         host[0:B].view(np.float32)[:] = [max(p.temperature, 0.0) for p in params]
         host[B : 2 * B].view(np.float32)[:] = [p.top_p for p in params]
         host[2 * B : 3 * B] = top_k
-        host[3 * B : 4 * B] = [s.num_output_tokens for s in seqs]
+        host[3 * B : 4 * B] = [s.num_output_tokens + ahead for s in seqs]
         host[4 * B :].view(np.int64)[:] = [_as_int64(s.noise_seed) for s in seqs]
         dev = torch.from_numpy(host).to(self.device, non_blocking=True)
         floats, ints = dev[: 2 * B].view(torch.float32), dev[2 * B : 4 * B]
         ops.sample(logits, floats[:B], ints[:B], floats[B:], dev[4 * B :].view(torch.int64), ints[B:], out,
                    max_top_k=max(kept))  # fmt: skip
-        return out.tolist()
+        return out
 
     def _apply_presence_penalty(self, logits, seqs):
         """Subtract each row's penalty from the logits of the tokens it has generated so far

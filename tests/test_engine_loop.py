@@ -125,3 +125,71 @@ def test_requests_without_a_seed_get_distinct_streams_and_seeded_ones_keep_their
     e._drain_inbox(block=False)
     a, b, c = e.scheduler.waiting
     assert a.noise_seed != b.noise_seed and c.noise_seed == 42
+
+
+class _LazyStep:
+    """A step of `AheadRunner` on its way: what it gives is worked out when it is read, from the
+    tokens that the sequences hold by then (a step sent ahead is read after the step before it)."""
+
+    device_tokens = None
+
+    def __init__(self, out, ahead):
+        self.out, self.ahead = out, ahead
+
+    def results(self):
+        if self.ahead:
+            return [StepResult([sum(s.token_ids) % 97], s.num_tokens) for s in self.out.seqs]
+        return [StepResult([sum(s.token_ids) % 97] if s.reaches_end(n) else [], s.num_computed_tokens + n)
+                for s, n in zip(self.out.seqs, self.out.num_new_tokens)]  # fmt: skip
+
+
+class AheadRunner(CountingRunner):
+    """The same tokens as `CountingRunner` through the interface of a runner that can send a decode
+    step to the GPU before the one before it was read."""
+
+    def __init__(self):
+        super().__init__()
+        self.sent_ahead = 0
+
+    def can_run_ahead(self, seqs):
+        return True
+
+    def launch(self, out, after=None):
+        self.calls += 1
+        self.sent_ahead += after is not None
+        if after is not None:  # what the engine promises for such a step
+            assert all(s.cache.tables[0] and len(s.cache.tables[0]) * 4 > s.num_tokens for s in out.seqs)
+            assert out.num_new_tokens == [1] * len(out.seqs)
+        return _LazyStep(out, after is not None)
+
+
+@pytest.mark.parametrize("eos", [frozenset(), frozenset({7, 23, 61})])
+def test_steps_sent_ahead_change_nothing_but_the_time(eos):
+    """With and without steps sent ahead: the same tokens and finish reasons, for requests that end on
+    a token, by length, at the longest sequence and by an abort in the middle; pages all given back."""
+    params = [SamplingParams(temperature=0.0, max_tokens=m, ignore_eos=False) for m in (10, 3, 25, 1, 17)]
+
+    def run(runner, **kw):
+        cfg = EngineConfig(**{"block_size": 4, "num_blocks": 64, "max_model_len": 24, **kw})
+        e = Engine(runner, Scheduler(cfg, eos))
+        handles = [e.submit(p, q) for p, q in zip(PROMPTS, params)]
+        steps = 0
+        while e.step():
+            steps += 1
+            if steps == 6:
+                e.abort(handles[2].id)
+                late = e.submit([3, 1, 4, 1, 5], params[0])  # arrives while others decode
+        handles.append(late)
+        outs = [(list(h), h.finish_reason) for h in handles]
+        assert e.stats()["kv_blocks_used"] == 0 and e._in_flight is None
+        return outs
+
+    plain = run(CountingRunner())
+    ahead_runner = AheadRunner()
+    assert run(ahead_runner) == plain
+    assert ahead_runner.sent_ahead >= 5
+    reasons = {reason for _, reason in plain}
+    assert {"length", "abort"} <= reasons and (not eos or "stop" in reasons)
+    # a pool so small that requests are preempted: steps go ahead only while nobody has to make room
+    tight = dict(num_blocks=10, max_num_seqs=3)
+    assert run(AheadRunner(), **tight) == run(CountingRunner(), **tight)

@@ -333,6 +333,50 @@ def test_greedy_generation_through_the_entry_point(setup, dtype):
                 seq.append(t)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_steps_sent_ahead_give_the_same_tokens(setup, dtype):
+    """While the running requests only decode, the engine sends the next step to the GPU before it has
+    read this one's tokens, and the GPU passes them on.  Seeded sampling, greedy rows, requests that
+    stop on a token, at their length and at the longest sequence, a request that arrives in the middle
+    and one that is aborted: token for token what the engine gives when it waits for every step."""
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.weights import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, dtype, "cuda:0")
+    vocab = raw["vocab_size"]
+    prompts = [rc.random_ids(vocab, n, seed=700 + n) for n in (3, 18, 40, 9, 26)]
+    params = [SamplingParams(temperature=0.8, top_k=12, top_p=0.9, max_tokens=30, seed=5),
+              SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True),
+              SamplingParams(temperature=1.0, top_k=0, top_p=1.0, max_tokens=60, seed=6),
+              SamplingParams(temperature=0.6, top_k=20, top_p=0.95, max_tokens=60, seed=7, ignore_eos=True),
+              SamplingParams(temperature=0.0, max_tokens=45)]  # fmt: skip
+    eos = frozenset(range(0, vocab, 9))  # a ninth of the vocabulary ends a request: some stop early
+
+    def run(run_ahead):
+        cfg = EngineConfig(block_size=16, num_blocks=64, max_model_len=64, max_num_seqs=8, max_num_batched_tokens=64)
+        engine = create_engine(model, cfg, eos)
+        engine.run_ahead = run_ahead
+        handles = [engine.submit(p, q) for p, q in zip(prompts, params)]
+        steps, sent = 0, 0
+        while engine.step():
+            steps += 1
+            sent += engine._in_flight is not None
+            if steps == 5:
+                engine.abort(handles[3].id)
+                handles.append(engine.submit(prompts[0][::-1] + prompts[1], params[0]))
+        assert engine.stats()["kv_blocks_used"] == 0
+        return [(list(h), h.finish_reason) for h in handles], sent
+
+    waited, none_sent = run(False)
+    ahead, sent = run(True)
+    assert none_sent == 0 and sent >= 10
+    assert ahead == waited
+    assert {reason for _, reason in waited} >= {"stop", "length", "abort"}
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_real_layer_sizes(dtype, tmp_path_factory):
     """Two layers of Qwen3-8B's sizes (hidden 4096, 32/8 heads of 128, intermediate 12288) with a
