@@ -377,6 +377,30 @@ def test_decode_steps_sent_ahead_give_the_same_tokens(setup, dtype):
     assert {reason for _, reason in waited} >= {"stop", "length", "abort"}
 
 
+def test_a_step_sent_ahead_may_be_the_first_of_its_graph(tmp_path):
+    """Requests that decode from 1,015 and 1,020 tokens pass the context bound of the captured steps
+    while steps are sent ahead: the step that is captured anew takes its tokens from the GPU like
+    any other, and the tokens are those of an engine that waits for every step."""
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.weights import load_model
+
+    raw = dict(TINY["A"], max_position_embeddings=2048)
+    weights = plain_random_weights(raw, seed=47, std=0.2, gain_std=0.2)
+    path = write_model_dir(str(tmp_path / "long"), raw, weights, torch.bfloat16)
+    model, _, _ = load_model(path, torch.float32, "cuda:0")
+    prompts = [rc.random_ids(raw["vocab_size"], n, seed=800 + n) for n in (1015, 1020)]
+    params = SamplingParams(temperature=0.7, top_k=10, max_tokens=24, seed=3, ignore_eos=True)
+    outs = []
+    for run_ahead in (False, True):
+        engine = create_engine(model, EngineConfig(block_size=16, num_blocks=160, max_model_len=1100, max_num_batched_tokens=2048))
+        engine.run_ahead = run_ahead
+        outs.append(engine.generate(prompts, params))
+        assert len(engine.runner.decode_graphs.graphs) == 2 and engine.stats()["kv_blocks_used"] == 0
+    assert outs[0] == outs[1] and all(len(o) == 24 for o in outs[0])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_real_layer_sizes(dtype, tmp_path_factory):
     """Two layers of Qwen3-8B's sizes (hidden 4096, 32/8 heads of 128, intermediate 12288) with a
