@@ -182,14 +182,16 @@ class Engine:
                 raise RuntimeError("scheduler has work but scheduled nothing")
             launch = getattr(self.runner, "launch", None)
             pending = launch(out) if launch is not None else None
+        sent = None
         if pending is None:
             results = self.runner.execute(out)
         else:
             ahead = self._plan_ahead(out)
             if ahead is not None:
-                self._in_flight = (ahead, self.runner.launch(ahead, after=pending))
+                sent = (ahead, self.runner.launch(ahead, after=pending))
             results = pending.results()
         new_tokens = self.scheduler.update(out, results)
+        self._in_flight = sent  # only now: a step that failed on the way leaves nothing behind
 
         now = time.perf_counter()
         self.num_steps += 1

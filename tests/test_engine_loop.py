@@ -156,6 +156,8 @@ class AheadRunner(CountingRunner):
 
     def launch(self, out, after=None):
         self.calls += 1
+        if self.fail_at is not None and self.calls >= self.fail_at:
+            raise RuntimeError("device fell over")
         self.sent_ahead += after is not None
         if after is not None:  # what the engine promises for such a step
             assert all(s.cache.tables[0] and len(s.cache.tables[0]) * 4 > s.num_tokens for s in out.seqs)
@@ -193,3 +195,19 @@ def test_steps_sent_ahead_change_nothing_but_the_time(eos):
     # a pool so small that requests are preempted: steps go ahead only while nobody has to make room
     tight = dict(num_blocks=10, max_num_seqs=3)
     assert run(AheadRunner(), **tight) == run(CountingRunner(), **tight)
+
+
+def test_a_failing_step_leaves_no_step_behind_it():
+    """The launch of a step sent ahead fails: the requests fail, nothing stays on its way, and the
+    engine serves the next request as if nothing had happened."""
+    e = Engine(AheadRunner(), Scheduler(EngineConfig(block_size=4, num_blocks=64, max_model_len=64), frozenset()))
+    e.runner.fail_at = 4  # the prompt, a decode step, one sent ahead, then the failure
+    e.start()
+    handle = e.submit([1, 2, 3], GREEDY)
+    with pytest.raises(RuntimeError, match="engine step failed"):
+        list(handle)
+    e.runner.fail_at = None
+    alone = engine().generate([[4, 5]], GREEDY)[0]
+    assert list(e.submit([4, 5], GREEDY)) == alone
+    e.shutdown()
+    assert e._in_flight is None and e.stats()["kv_blocks_used"] == 0 and e.runner.sent_ahead > 2
