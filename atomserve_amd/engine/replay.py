@@ -55,6 +55,10 @@ class Replay:
             if rid in seen:
                 raise ValueError(f"request {rid!r} appears twice in one step")
             seen.add(rid)
+            if not tokens:  # an entry that brings nothing runs nothing
+                if want:
+                    raise ValueError(f"request {rid!r} wants logits of a step in which it has no tokens")
+                continue
             if rid not in self.live:
                 self.live[rid] = [self.manager.new_request(), 0]
             rc, computed = self.live[rid]
@@ -70,9 +74,10 @@ class Replay:
             if out.shape[0]:
                 logits = out.cpu()
             for e in entries:
-                state = self.live[e["id"]]
-                state[1] += len(e["tokens"])
-                self.manager.release_behind_window(state[0], state[1])
+                if e["tokens"]:
+                    state = self.live[e["id"]]
+                    state[1] += len(e["tokens"])
+                    self.manager.release_behind_window(state[0], state[1])
         for rid in end:
             if rid in self.live:
                 self.manager.release(self.live.pop(rid)[0])

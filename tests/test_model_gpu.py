@@ -270,8 +270,10 @@ def test_trace_run_program(setup, dtype, tmp_path):
     other = rc.random_ids(raw["vocab_size"], 21, seed=4)
     steps = [
         {"step": 0, "entries": [{"id": "a", "tokens": ids[:30], "want": [0, 29]}], "end": []},
-        {"step": 1, "entries": [{"id": "a", "tokens": ids[30:33], "want": []}, {"id": "b", "tokens": other, "want": [20]}], "end": ["b"]},
+        {"step": 1, "entries": [{"id": "a", "tokens": ids[30:33], "want": []}, {"id": "c", "tokens": [], "want": []},
+                                {"id": "b", "tokens": other, "want": [20]}], "end": ["b"]},  # fmt: skip
         {"step": 2, "entries": [{"id": "a", "tokens": ids[33:], "want": [16]}], "end": ["a"]},
+        {"step": 3, "entries": [], "end": ["c"]},  # nothing to run, nothing to write
     ]
     out = tmp_path / "out"
     proc = subprocess.run(
@@ -280,7 +282,8 @@ def test_trace_run_program(setup, dtype, tmp_path):
         input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
     )  # fmt: skip
     assert proc.returncode == 0, proc.stderr[-2000:]
-    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2"]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
+    assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "2.f32"]
     ref_a, ref_b = plain.logits(raw, weights, ids).float().numpy(), plain.logits(raw, weights, other).float().numpy()
     got0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1)
     got1 = np.fromfile(out / "1.f32", dtype="<f4").reshape(1, -1)
