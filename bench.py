@@ -50,6 +50,8 @@ def parse_args():
     p.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     p.add_argument("--points", default="1,64", help="other decode batch sizes to measure (fewer steps each)")
     p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt whose prefill is timed "
+                   "(longer than 2,048: in steps of 2,048 tokens)")  # fmt: skip
     p.add_argument("--no-calibration", action="store_true", help="skip the library copy and matmul probes")
     p.add_argument("--greedy", action="store_true", help="greedy instead of the default sampling settings")
     p.add_argument("--workload", choices=["decode", "mixed"], default="decode",
@@ -187,7 +189,7 @@ def main() -> int:
 
     batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
     block = 16
-    max_len = max(args.max_len, args.context + args.steps + args.warmup + 16)
+    max_len = max(args.max_len, args.context + args.steps + args.warmup + 16, args.prefill_tokens + 16)
     num_blocks = max(batches) * max_len // block
     params = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True) if args.greedy else \
         SamplingParams(max_tokens=100000, ignore_eos=True)  # fmt: skip
@@ -229,7 +231,7 @@ def main() -> int:
     result_prefill = None
     if not args.no_prefill:
         one = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
-        T = 2048
+        T = args.prefill_tokens
         for i in range(2):  # warm-up: libraries pick their kernels, pools are touched
             engine.generate([prompt(99 - i, T, c.vocab_size)], one)
         times = []
