@@ -49,6 +49,7 @@ def parse_args():
     p.add_argument("--max-len", type=int, default=4096, help="longest sequence the cache pool is sized for")
     p.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     p.add_argument("--points", default="1,64", help="other decode batch sizes to measure (fewer steps each)")
+    p.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt whose prefill is timed "
                    "(longer than 2,048: in steps of 2,048 tokens)")  # fmt: skip
@@ -188,7 +189,7 @@ def main() -> int:
         return 0
 
     batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
-    block = 16
+    block = args.block_size
     max_len = max(args.max_len, args.context + args.steps + args.warmup + 16, args.prefill_tokens + 16)
     num_blocks = max(batches) * max_len // block
     params = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True) if args.greedy else \
