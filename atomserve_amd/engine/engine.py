@@ -211,15 +211,17 @@ class Engine:
 
     def _plan_ahead(self, out):
         """The decode step after `out`, if it is certain but for its tokens: `out` gives every running
-        request a token, nobody waits or has left, nobody reaches its length with that token, no sampling
+        request a token, nobody can be admitted or has left, nobody reaches its length with that token, no sampling
         setting needs the tokens on the host, and every request has a page for one more position.  A
         request that ends on an end-of-sequence token in `out` still takes part in the step ahead; its
         result there is dropped and its pages, given back at once, may be written once more, which is
         harmless: whoever gets them next writes after that, in the order of the GPU's queue."""
         s = self.scheduler
         can = getattr(self.runner, "can_run_ahead", None)
-        if not self.run_ahead or can is None or out.preempted or s.waiting or not self._inbox.empty():
+        if not self.run_ahead or can is None or out.preempted or not self._inbox.empty():
             return None
+        if s.waiting and len(s.running) < s.config.max_num_seqs:
+            return None  # somebody may be admitted next; with every place taken the queue just waits on
         if len(out.seqs) != len(s.running) or any(a is not b for a, b in zip(out.seqs, s.running)):
             return None
         limit = s.config.max_model_len

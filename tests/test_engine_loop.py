@@ -195,6 +195,16 @@ def test_steps_sent_ahead_change_nothing_but_the_time(eos):
     # a pool so small that requests are preempted: steps go ahead only while nobody has to make room
     tight = dict(num_blocks=10, max_num_seqs=3)
     assert run(AheadRunner(), **tight) == run(CountingRunner(), **tight)
+    # every place taken and a queue behind: the queue cannot move, so steps still go ahead
+    # (a request that ends on a token leaves its place one step later then, so the abort at the sixth
+    # step finds its request a token further or less: that one is compared up to the shorter reply)
+    full = AheadRunner()
+    ahead, waited = run(full, max_num_seqs=2), run(CountingRunner(), max_num_seqs=2)
+    assert full.sent_ahead >= 5
+    assert ahead[:2] + ahead[3:] == waited[:2] + waited[3:]
+    (a, reason_a), (w, reason_w) = ahead[2], waited[2]
+    n = min(len(a), len(w))
+    assert a[:n] == w[:n] and reason_a == reason_w == "abort"
 
 
 def test_a_failing_step_leaves_no_step_behind_it():
