@@ -154,11 +154,6 @@ class DecodeGraphs:
         return len(self.graphs) - before
 
 
-class _Passed:
-    def synchronize(self) -> None:
-        pass
-
-
 class PendingStep:
     """A step that is on the GPU, sampling included; `results()` waits for its tokens."""
 
@@ -246,17 +241,15 @@ class ModelRunner:
         device_tokens = self.sampler.launch(logits, sampling, ahead=0 if after is None else 1)
         host_tokens = event = None
         if device_tokens is not None:
-            if device_tokens.is_cuda:
-                if len(self._token_buffers) < 3:
-                    self._token_buffers.append(torch.empty(4096, dtype=torch.int32, pin_memory=True))
-                self._token_turn = (self._token_turn + 1) % len(self._token_buffers)
-                host_tokens = self._token_buffers[self._token_turn]
-                if host_tokens.numel() < device_tokens.shape[0]:
-                    host_tokens = self._token_buffers[self._token_turn] = torch.empty(
-                        device_tokens.shape[0], dtype=torch.int32, pin_memory=True)  # fmt: skip
-                host_tokens[: device_tokens.shape[0]].copy_(device_tokens, non_blocking=True)
-                event = torch.cuda.Event()
-                event.record()
-            else:
-                host_tokens, event = device_tokens, _Passed()
+            # three pinned buffers in turn: at most two steps are on their way at any time
+            if len(self._token_buffers) < 3:
+                self._token_buffers.append(torch.empty(4096, dtype=torch.int32, pin_memory=True))
+            self._token_turn = (self._token_turn + 1) % len(self._token_buffers)
+            host_tokens = self._token_buffers[self._token_turn]
+            if host_tokens.numel() < device_tokens.shape[0]:
+                host_tokens = self._token_buffers[self._token_turn] = torch.empty(
+                    device_tokens.shape[0], dtype=torch.int32, pin_memory=True)  # fmt: skip
+            host_tokens[: device_tokens.shape[0]].copy_(device_tokens, non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
         return PendingStep(samples, num_computed, device_tokens, host_tokens, event)
