@@ -179,6 +179,19 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
 ATTN_FILL_GROUPS = 512  # (token, kv head) pairs that occupy every compute unit twice over
 
 
+MFMA_PARTITIONS = (128, 256, 512, 1024, 2048)  # keys per workgroup of the matrix-core decode kernel
+
+
+def _partition_cost(groups: int, span: int, part: int) -> float:
+    """Microseconds, roughly, of the decode attention and its merge when `groups` (token, kv head) pairs
+    cut `span` keys into partitions of `part`: a workgroup costs 4 us and 25 ns a key, 512 of them run
+    at a time, and the merge 0.6 us a partition.  Fitted to the kernel's times at 1 to 32 requests of
+    500 to 33,000 keys (heads of 128, 8 kv heads); what it picks is within 2 per cent of the best
+    partition size on average there, where one size for all was 8 per cent off."""
+    parts = math.ceil(span / part)
+    return (4.0 + 0.025 * min(part, span)) * max(1.0, groups * parts / 512) + 0.6 * parts
+
+
 def _partitions(N, H, KV, D, max_context, window, mfma, part_size, device):
     """How the keys of N single queries are cut for the split-KV kernels, and the buffers of the
     partial results: (part_size, P, part_m, part_l, part_acc), the buffers None when P == 1."""
@@ -188,15 +201,15 @@ def _partitions(N, H, KV, D, max_context, window, mfma, part_size, device):
         # Enough partitions to occupy the GPU when few tokens are in the batch, few enough that
         # the merge stays small; boundaries are multiples of part_size in absolute position.
         if mfma:
-            groups, part_size = N * KV, 128  # 4 waves x 32 keys: one round of loads per workgroup
-            limit = 1024
+            groups = N * KV
+            if groups >= ATTN_FILL_GROUPS:
+                part_size = -(-span // 32) * 32  # enough workgroups without partitions: no merge
+            else:
+                part_size = min(MFMA_PARTITIONS, key=lambda part: _partition_cost(groups, span, part))
         else:
             groups, part_size = N * KV * max(1, (G + 7) // 8), 256
-            limit = 2048
-        while part_size < span and groups * math.ceil(span / part_size) > limit:
-            part_size *= 2
-        if mfma and groups >= ATTN_FILL_GROUPS:
-            part_size = max(part_size, -(-span // 32) * 32)  # enough workgroups without partitions: no merge
+            while part_size < span and groups * math.ceil(span / part_size) > 2048:
+                part_size *= 2
     if mfma and part_size % 32:
         raise KernelError("attention: partitions of the matrix-core kernel are multiples of 32 keys")
     P = max(1, math.ceil(max_context / part_size))
