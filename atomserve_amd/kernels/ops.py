@@ -176,7 +176,7 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
-ATTN_FILL_GROUPS = 512  # (token, kv head) pairs that occupy every compute unit twice over
+ATTN_FILL_GROUPS = 384  # (token, kv head) pairs from which on whole contexts beat partitions and their merge (measured)
 
 
 MFMA_PARTITIONS = (128, 256, 512, 1024, 2048)  # keys per workgroup of the matrix-core decode kernel
