@@ -466,6 +466,15 @@ def _fastest_of(trial) -> int:
 GATED_MAX_K = 6144  # the widest input the fused product-and-activation kernel keeps in registers
 
 
+GATED_TWO_TILES = True
+
+
+def _gated_two_tiles(rows: int, k: int) -> bool:
+    """17 to 32 rows through the gated kernel with two row tiles also where the plain products of such
+    widths are the library's: it saves the activation kernel and the write and read of gate and up."""
+    return GATED_TWO_TILES and SKINNY_MAX_ROWS < rows <= SKINNY_TWO_MAX_ROWS and k <= SKINNY_TWO_MAX_K and k % 8 == 0
+
+
 def gemm_silu_mul(a, w, out) -> None:
     """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for w[2 I, K]: the gate and up products and
     the activation.  bf16 with few rows: one kernel, the products rounded to bf16 before the
@@ -477,7 +486,7 @@ def gemm_silu_mul(a, w, out) -> None:
     _check(w, "w", a.dtype, (2 * inter, K))
     if M == 0:
         return
-    if a.dtype == BF16 and _few_rows(M, K, inter, GATED_MAX_K):
+    if a.dtype == BF16 and (_few_rows(M, K, inter, GATED_MAX_K) or _gated_two_tiles(M, K)):
         call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), M, inter, K, _stream())
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
