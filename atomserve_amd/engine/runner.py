@@ -51,10 +51,10 @@ class DecodeGraphs:
     correctly (checked against eager steps in the tests, several replays with eager work between).
 
     All captured steps draw their intermediate tensors from one memory pool (they never run at the
-    same time), so a step holds only its own logits beyond it, 39 MB for 64 rows of a 152K
+    same time), so a step holds only its own logits beyond it, 39 MB for 64 rows (155 MB for 256) of a 152K
     vocabulary; at most `MAX_GRAPHS` are kept, the one replayed longest ago goes first."""
 
-    ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64)
+    ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
     CONTEXT_STEP = 1024
     MAX_GRAPHS = 64
 

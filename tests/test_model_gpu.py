@@ -148,7 +148,7 @@ def test_decoding_across_the_context_bound_of_a_captured_graph(dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("num_requests", [3, 13, 21, 40])
+@pytest.mark.parametrize("num_requests", [3, 13, 21, 40, 100])
 def test_decode_graphs_replay_what_eager_steps_give(setup, dtype, num_requests):
     """Decode steps replayed as captured graphs against the same steps launched kernel by kernel:
     the same logits at every step, over several replays with eager work (a new request's prompt)
