@@ -168,3 +168,96 @@ def test_sampling_distribution_rules():
     assert (plain.sampling_distribution(row, 1.0, 0, 0.01) > 0).tolist() == [True, False, False, False]
     sharp = plain.sampling_distribution(row, 0.5, 0, 1.0)
     assert torch.allclose(sharp, probs**2 / (probs**2).sum())
+
+
+def test_batched_attention_is_the_loop_form():
+    # groups of 3, a window, queries that start past the first keys, keys at given positions
+    q, k, v = torch.randn(9, 6, 8, dtype=F64), torch.randn(14, 2, 8, dtype=F64), torch.randn(14, 2, 8, dtype=F64)
+    for window in (0, 4):
+        loop = plain.causal_attention(q, k, v, torch.arange(5, 14), window=window)
+        for rows in (512, 4):
+            batched = plain.causal_attention_batched(q, k, v, torch.arange(5, 14), window=window, rows=rows)
+            assert torch.allclose(batched, loop, atol=1e-12)
+    kp = torch.arange(100, 114)
+    assert torch.allclose(plain.causal_attention_batched(q, k, v, torch.arange(105, 114), k_positions=kp),
+                          plain.causal_attention(q, k, v, torch.arange(105, 114), k_positions=kp), atol=1e-12)
+    raw = TINY_B
+    w = plain_random_weights(raw, seed=4, std=0.2, gain_std=0.2)
+    ids = torch.randint(0, raw["vocab_size"], (17,)).tolist()
+    assert torch.allclose(plain.logits(raw, w, ids, batched=True), plain.logits(raw, w, ids), atol=1e-10)
+
+
+def _library_head(raw, w, x):
+    head = w["model.embed_tokens.weight" if raw["tie_word_embeddings"] else "lm_head.weight"].to(F64)
+    h = raw["hidden_size"]
+    return F.linear(F.rms_norm(x, (h,), w["model.norm.weight"].to(F64), raw["rms_norm_eps"]), head)
+
+
+@pytest.mark.parametrize("raw", [TINY_A, TINY_B])
+def test_without_mixer_and_feed_forward_the_model_is_embedding_norm_head(raw):
+    # With o_proj and down_proj zeroed every layer adds nothing: what remains is the unscaled
+    # embedding, the final norm on the stream, and the head.  An embedding multiplier, a missing
+    # final norm or a head bias would show.
+    w = plain_random_weights(raw, seed=6, std=0.2, gain_std=0.3)
+    for name in w:
+        if name.endswith("o_proj.weight") or name.endswith("down_proj.weight"):
+            w[name] = torch.zeros_like(w[name])
+    ids = torch.randint(0, raw["vocab_size"], (9,))
+    x = w["model.embed_tokens.weight"].to(F64)[ids]
+    assert torch.allclose(plain.logits(raw, w, ids.tolist()), _library_head(raw, w, x), atol=1e-10)
+
+
+@pytest.mark.parametrize("raw", [TINY_A, TINY_B])
+def test_layer_arrangement_against_library_routines(raw):
+    # The whole arrangement spelled with library routines only: x += attn(norm_in(x));
+    # x += mlp(norm_post(x)), each norm read from the un-normalised stream and each sum taken on
+    # it.  Post-norm, a residual taken from the normalised rows, swapped norm gains or a
+    # feed-forward fed by the attention's input would each change the result by far more than 1e-9.
+    raw = dict(raw)
+    w = plain_random_weights(raw, seed=8, std=0.25, gain_std=0.4)
+    wd = {k: v.to(F64) for k, v in w.items()}
+    T, h = 10, raw["hidden_size"]
+    H, KV, D = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
+    eps, theta = raw["rms_norm_eps"], raw["rope_theta"]
+    ids = torch.randint(0, raw["vocab_size"], (T,))
+    pos = torch.arange(T)
+    x = wd["model.embed_tokens.weight"][ids]
+    for i in range(raw["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        a = F.rms_norm(x, (h,), wd[p + "input_layernorm.weight"], eps)
+        q = F.rms_norm(F.linear(a, wd[p + "self_attn.q_proj.weight"]).view(T, H, D), (D,), wd[p + "self_attn.q_norm.weight"], eps)
+        k = F.rms_norm(F.linear(a, wd[p + "self_attn.k_proj.weight"]).view(T, KV, D), (D,), wd[p + "self_attn.k_norm.weight"], eps)
+        v = F.linear(a, wd[p + "self_attn.v_proj.weight"]).view(T, KV, D)
+        q, k = plain.rope(q, pos, theta), plain.rope(k, pos, theta)  # pinned above by vectors and complex products
+        g = H // KV
+        o = F.scaled_dot_product_attention(q.transpose(0, 1), k.repeat_interleave(g, 1).transpose(0, 1),
+                                           v.repeat_interleave(g, 1).transpose(0, 1), is_causal=True)
+        x = x + F.linear(o.transpose(0, 1).reshape(T, H * D), wd[p + "self_attn.o_proj.weight"])
+        m = F.rms_norm(x, (h,), wd[p + "post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(m, wd[p + "mlp.gate_proj.weight"])) * F.linear(m, wd[p + "mlp.up_proj.weight"]),
+                         wd[p + "mlp.down_proj.weight"])
+    assert torch.allclose(plain.logits(raw, w, ids.tolist()), _library_head(raw, w, x), atol=1e-9)
+
+
+def test_one_sublayer_at_a_time_reads_the_stream_not_the_normalised_rows():
+    # One layer with the attention silenced: logits = head(norm(e + mlp(norm_post(e)))).  With the
+    # feed-forward silenced instead: head(norm(e + attn(norm_in(e)))) where a single token attends
+    # to itself alone, so attn is o_proj(v_proj(norm_in(e))): no softmax, rotation or q/k norm enters.
+    raw = dict(TINY_B, num_hidden_layers=1)
+    w = plain_random_weights(raw, seed=10, std=0.25, gain_std=0.4)
+    wd = {k: v.to(F64) for k, v in w.items()}
+    p, h, eps = "model.layers.0.", raw["hidden_size"], raw["rms_norm_eps"]
+    e = wd["model.embed_tokens.weight"][torch.tensor([7])]
+    silent = dict(w)
+    silent[p + "self_attn.o_proj.weight"] = torch.zeros_like(w[p + "self_attn.o_proj.weight"])
+    m = F.rms_norm(e, (h,), wd[p + "post_attention_layernorm.weight"], eps)
+    mlp = F.linear(F.silu(F.linear(m, wd[p + "mlp.gate_proj.weight"])) * F.linear(m, wd[p + "mlp.up_proj.weight"]),
+                   wd[p + "mlp.down_proj.weight"])
+    assert torch.allclose(plain.logits(raw, silent, [7]), _library_head(raw, w, e + mlp), atol=1e-10)
+    silent = dict(w)
+    silent[p + "mlp.down_proj.weight"] = torch.zeros_like(w[p + "mlp.down_proj.weight"])
+    a = F.rms_norm(e, (h,), wd[p + "input_layernorm.weight"], eps)
+    g = raw["num_attention_heads"] // raw["num_key_value_heads"]
+    v = F.linear(a, wd[p + "self_attn.v_proj.weight"]).view(1, raw["num_key_value_heads"], raw["head_dim"])
+    attn = F.linear(v.repeat_interleave(g, 1).reshape(1, -1), wd[p + "self_attn.o_proj.weight"])
+    assert torch.allclose(plain.logits(raw, silent, [7]), _library_head(raw, w, e + attn), atol=1e-10)
