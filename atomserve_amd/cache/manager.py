@@ -121,6 +121,23 @@ class CacheManager:
             rc.state_slot = self._free_slots.pop()
         return True
 
+    def reserve_all(self, wanted) -> bool:
+        """`reserve` for several requests of one step together: wanted = [(rc, num_computed, num_new)],
+        each request at most once.  All or nothing: on False no request has taken anything."""
+        short = [0] * len(self.paged_groups)
+        slots = 0
+        for rc, num_computed, num_new in wanted:
+            need = blocks_for_tokens(num_computed + num_new, self.block_size)
+            for g, table in enumerate(rc.tables):
+                short[g] += max(0, need - len(table))
+            slots += 1 if self.state_groups and rc.state_slot < 0 else 0
+        if any(m > g.allocator.num_free for g, m in zip(self.paged_groups, short)) or slots > len(self._free_slots):
+            return False
+        for rc, num_computed, num_new in wanted:
+            if not self.reserve(rc, num_computed, num_new):
+                raise RuntimeError("pages counted as free could not be taken")
+        return True
+
     def release_behind_window(self, rc: RequestCache, num_computed: int) -> int:
         """Give back the pages of windowed groups that no query at a position >= num_computed
         can see any more.  Returns how many pages were freed."""

@@ -357,7 +357,22 @@ def gemm(a, w, out) -> None:
 LIBRARY_WORKSPACE_BYTES = 64 << 20
 LIBRARY_TUNED_ROWS = {32, 64}
 LIBRARY_TRIALS_EACH = 4
-_library = {"workspace": None, "choice": {}, "trials": {}}
+_library = {"workspace": None, "choice": {}, "trials": {}, "fixed": False}
+
+
+def fix_library_choices(fixed: bool = True) -> None:
+    """fixed: every shape not settled yet takes the library's first candidate (what torch.mm runs)
+    instead of timing the candidates, so that bfloat16 results are the same from process to process.
+    Choices already made stay (they were made under the setting of their time)."""
+    _library["fixed"] = bool(fixed)
+    if fixed:
+        _library["trials"].clear()
+
+
+def library_choices() -> dict:
+    """(rows, columns, width, output dtype) -> the candidate that runs, for every shape settled so far
+    (-1: torch's own call); enough to reproduce a run's products."""
+    return dict(_library["choice"])
 
 
 def _torch_gemm(a, w, out) -> None:
@@ -382,7 +397,7 @@ def _library_gemm(a, w, out, M, N, K) -> None:
             count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
             if count == 0:
                 choice = state["choice"][key] = -1  # the library offers nothing for this shape through this door
-            elif count == 1 or M not in LIBRARY_TUNED_ROWS:
+            elif count == 1 or M not in LIBRARY_TUNED_ROWS or state["fixed"]:
                 choice = state["choice"][key] = 0  # the library's first candidate, which is what torch.mm runs
             else:
                 trial = state["trials"][key] = {"count": count, "runs": []}

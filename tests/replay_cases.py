@@ -38,16 +38,18 @@ def portions(rid, ids, sizes=(9, 2, 17, 3, 2, 31, 8, 5, 64, 2, 11)):
     return steps
 
 
-def mixed(requests: dict, seed=0, max_live=4, prompt_fraction=0.6, sizes=(2, 7, 19, 3, 33, 12)):
+def mixed(requests: dict, seed=0, max_live=4, prompt_fraction=0.6, sizes=(2, 7, 19, 3, 33, 12), prompt_lengths=None):
     """Up to `max_live` requests at a time: portions of some prompts beside single tokens of
-    others; a request's turn may be skipped; new ones start as old ones end."""
+    others; a request's turn may be skipped; new ones start as old ones end.
+    prompt_lengths: request id -> how many of its tokens come in portions (default: a fraction)."""
     rng = random.Random(seed)
     waiting = list(requests.items())
     live, steps = {}, []
     while waiting or live:
         while waiting and len(live) < max_live:
             rid, ids = waiting.pop(0)
-            live[rid] = {"ids": ids, "at": 0, "prompt": max(2, int(len(ids) * prompt_fraction))}
+            prompt = (prompt_lengths or {}).get(rid, int(len(ids) * prompt_fraction))
+            live[rid] = {"ids": ids, "at": 0, "prompt": max(2, prompt)}
         entries, end = [], []
         for rid, st in list(live.items()):
             if len(live) > 1 and rng.random() < 0.15:
@@ -84,8 +86,9 @@ def live_token_bound(steps, unit=64):
     return worst
 
 
-def run_and_compare(replay, steps, requests: dict, raw, weights, reference_cache: dict):
-    """Feed `steps` to a `Replay`; returns (largest |difference|, largest |reference|, rows compared)."""
+def run_and_compare(replay, steps, requests: dict, raw, weights, reference_cache: dict, plain_kwargs=None):
+    """Feed `steps` to a `Replay`; returns (largest |difference|, largest |reference|, rows compared).
+    plain_kwargs: how the plain model runs (default: float64 on the CPU, the loop form)."""
     at = {rid: 0 for rid in requests}
     worst, scale, rows = 0.0, 0.0, 0
     for s in steps:
@@ -94,7 +97,7 @@ def run_and_compare(replay, steps, requests: dict, raw, weights, reference_cache
         for e in s["entries"]:
             rid = e["id"]
             if rid not in reference_cache:
-                reference_cache[rid] = plain.logits(raw, weights, requests[rid]).float()
+                reference_cache[rid] = plain.logits(raw, weights, requests[rid], **(plain_kwargs or {})).float().cpu()
             ref = reference_cache[rid]
             for w in e["want"]:
                 got = logits[k]

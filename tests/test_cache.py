@@ -195,3 +195,34 @@ def test_prefix_adoption_stops_at_the_first_miss_and_leaves_a_token():
         m.release(rc)
     assert m.num_free == 16 and m.num_cached == 2
     m.check()
+
+
+def test_reserving_for_a_whole_step_is_all_or_nothing():
+    from atomserve_amd.cache.manager import CacheManager
+    from atomserve_amd.parts.base import PagedCacheRequest, StateCacheRequest
+
+    m = CacheManager({0: PagedCacheRequest(2, 16), 1: StateCacheRequest((4,))}, block_size=4, num_blocks=6, max_num_seqs=2)
+    a, b, c = m.new_request(), m.new_request(), m.new_request()
+    assert m.reserve_all([(a, 0, 9), (b, 0, 10)])  # 3 + 3 pages, both slots
+    assert m.num_free == 0 and a.state_slot >= 0 and b.state_slot >= 0 and a.state_slot != b.state_slot
+    assert m.reserve_all([(a, 9, 3), (b, 10, 2)])  # both fit in the pages they hold
+    before = ([list(t) for t in a.tables], [list(t) for t in b.tables])
+    assert not m.reserve_all([(a, 12, 1), (b, 12, 0)])  # a needs a fourth page: nobody gets anything
+    assert ([list(t) for t in a.tables], [list(t) for t in b.tables]) == before
+    m.release(b)
+    assert not m.reserve_all([(a, 12, 1), (b, 0, 4), (c, 0, 1)])  # pages would do, slots would not
+    assert m.num_free == 3 and b.state_slot < 0 and c.state_slot < 0
+    assert m.reserve_all([(a, 12, 1), (b, 0, 4)])
+    m.release(a)
+    m.release(b)
+    assert m.num_free == 6 and m.num_free_slots == 2
+    m.check()
+
+
+def test_pages_of_a_replay_pool():
+    from atomserve_amd.engine.replay import pages_for
+
+    assert pages_for(256, 16, 4) == 16 and pages_for(256, 8, 4) == 32 and pages_for(256, 64, 4) == 4
+    # pages that do not divide 64: four requests of 64 tokens take two pages of 48 each
+    assert pages_for(256, 48, 4) >= 8 and pages_for(256, 128, 4) >= 4
+    assert pages_for(0, 16, 4) == 1

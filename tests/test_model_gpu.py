@@ -20,6 +20,7 @@ pytestmark = pytest.mark.gpu
 # bf16: activations carry 8 bits; the bound is a few rounding steps of the largest logit.
 TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 LENGTHS = {"A": 200, "B": 420}
+PAGE = {"A": 16, "B": 8}  # each tiny configuration at its own page size
 
 
 @pytest.fixture(scope="module", params=["A", "B"])
@@ -31,10 +32,10 @@ def setup(request, tmp_path_factory):
     return name, raw, weights, path, {}
 
 
-def make_replay(path, dtype, max_tokens):
+def make_replay(path, dtype, max_tokens, block_size=16, max_live=4):
     from atomserve_amd.engine.replay import Replay
 
-    return Replay(path, dtype, max_tokens)
+    return Replay(path, dtype, max_tokens, block_size=block_size, max_live=max_live)
 
 
 def check(worst, scale, dtype):
@@ -47,7 +48,7 @@ def test_whole_decoded_and_in_portions(setup, dtype):
     ids = rc.random_ids(raw["vocab_size"], LENGTHS[name], seed=1)
     requests = {"a": ids}
     for steps in (rc.whole("a", ids), rc.prefill_then_decode("a", ids), rc.portions("a", ids)):
-        replay = make_replay(path, dtype, rc.live_token_bound(steps))
+        replay = make_replay(path, dtype, rc.live_token_bound(steps), PAGE[name])
         worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
         assert rows >= 33
         check(worst, scale, dtype)
@@ -62,11 +63,31 @@ def test_mixed_requests_with_pages_used_again(setup, dtype):
     steps = rc.mixed(requests, seed=5)
     bound = rc.live_token_bound(steps)
     assert bound < sum(-(-n // 64) * 64 for n in lengths)  # fewer pages than all requests need: reuse
-    replay = make_replay(path, dtype, bound)
+    replay = make_replay(path, dtype, bound, PAGE[name])
     worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
     assert rows > 200
     check(worst, scale, dtype)
     assert replay.manager.num_free == replay.manager.num_blocks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("block_size", [8, 16, 32, 48])
+def test_every_cut_at_other_page_sizes(setup, dtype, block_size):
+    """Whole, decoded, in portions and mixed with pages used again, at pages of 8, 16, 32 and 48
+    tokens (48 divides neither the 64 queries of a tile nor the 64 tokens that the pool is counted
+    in; 8 sends bfloat16 through the general attention kernel): the same logits."""
+    name, raw, weights, path, cache = setup
+    lengths = [70, 33, 150, 64, 97, 20] if name == "A" else [90, 300, 64, 17, 257, 128]
+    requests = {f"r{i}": rc.random_ids(raw["vocab_size"], n, seed=100 + i) for i, n in enumerate(lengths)}
+    first = ("r2", requests["r2"])
+    mixed = rc.mixed(requests, seed=block_size)
+    assert rc.live_token_bound(mixed) < sum(-(-n // 64) * 64 for n in lengths)
+    for steps in (rc.whole(*first), rc.prefill_then_decode(*first), rc.portions(*first), mixed):
+        replay = make_replay(path, dtype, rc.live_token_bound(steps), block_size)
+        worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
+        assert rows >= 33
+        check(worst, scale, dtype)
+        assert replay.manager.num_free == replay.manager.num_blocks
 
 
 @pytest.mark.parametrize("seed", range(6))
@@ -84,7 +105,7 @@ def test_random_traces_in_32_bit(setup, seed):
                 for i in range(rng.randint(2, 7))}  # fmt: skip
     sizes = tuple(rng.choice([2, 3, 5, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100]) for _ in range(6))
     steps = rc.mixed(requests, seed=seed, max_live=rng.randint(1, 4), prompt_fraction=rng.choice([0.3, 0.6, 0.95]), sizes=sizes)
-    replay = make_replay(path, "float32", rc.live_token_bound(steps))
+    replay = make_replay(path, "float32", rc.live_token_bound(steps), rng.choice([4, 8, 16, 24, 64]))
     worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, {})
     assert rows > 0 and worst <= 0.3 * TOL["float32"] * max(scale, 1.0)
     assert replay.manager.num_free == replay.manager.num_blocks
@@ -112,9 +133,10 @@ def test_configurations_drawn_at_random(seed, tmp_path):
     first = next(iter(requests.items()))
     cases = [rc.whole(*first), rc.prefill_then_decode(*first), rc.portions(*first), rc.mixed(requests, seed=seed)]
     cache = {}
+    page = rng.choice([8, 16, 32, 48, 64])
     for dtype in ("float32", "bfloat16"):
         for steps in cases:
-            replay = make_replay(path, dtype, rc.live_token_bound(steps))
+            replay = make_replay(path, dtype, rc.live_token_bound(steps), page)
             worst, scale, rows = rc.run_and_compare(replay, steps, requests, raw, weights, cache)
             assert rows > 0 and replay.manager.num_free == replay.manager.num_blocks
             check(worst, scale, dtype)
@@ -126,7 +148,7 @@ def test_first_tokens_and_long_decoding(setup, dtype):
     n = LENGTHS[name]
     ids = rc.random_ids(raw["vocab_size"], n, seed=2)
     steps = [{"step": i, "entries": [{"id": "d", "tokens": [ids[i]], "want": [0]}], "end": []} for i in range(n)]
-    replay = make_replay(path, dtype, n + 64)
+    replay = make_replay(path, dtype, n + 64, PAGE[name])
     worst, scale, rows = rc.run_and_compare(replay, steps, {"d": ids}, raw, weights, cache)
     assert rows == n
     check(worst, scale, dtype)
@@ -276,10 +298,13 @@ def test_trace_run_program(setup, dtype, tmp_path):
         {"step": 3, "entries": [], "end": ["c"]},  # nothing to run, nothing to write
     ]
     out = tmp_path / "out"
+    # the cache's geometry comes with the trace (a first line) or on the command line
+    header = [{"geometry": {"block_size": 8, "pages": 16, "max_live": 3}}] if name == "B" else []
+    geometry_flags = [] if name == "B" else ["--block-size", "32", "--max-live", "3"]
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", path, "--dtype", dtype, "--out", str(out),
-         "--max-tokens", "128"],
-        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
+         "--max-tokens", "128", *geometry_flags],
+        input="\n".join(json.dumps(s) for s in header + steps) + "\n", capture_output=True, text=True, timeout=600,
     )  # fmt: skip
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
@@ -366,7 +391,7 @@ def test_decode_steps_sent_ahead_give_the_same_tokens(setup, dtype):
         steps, sent = 0, 0
         while engine.step():
             steps += 1
-            sent += engine._in_flight is not None
+            sent += engine.steps_in_flight > 0
             if steps == 5:
                 engine.abort(handles[3].id)
                 handles.append(engine.submit(prompts[0][::-1] + prompts[1], params[0]))
