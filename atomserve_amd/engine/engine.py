@@ -1,17 +1,22 @@
-"""The engine: one loop that owns the GPU (reference atomserve/engine.py:1-264).
+"""The engine: a pipeline of steps between the clients' queues and the GPU.
 
-    take new requests and aborts from the inbox -> scheduler
-    plan    = scheduler.schedule()
-    results = runner.execute(plan)        one pass over the GPU and one sampling call
-    scheduler.update(plan, results)
-    push each new token to its request's handle
+A step passes three stages, and one record (`_Flight`) carries it through them:
 
-While nothing changes among the running requests (all decode, nobody waits, nobody reaches its
-length), the next decode step goes to the GPU before this one's tokens are read: the GPU passes
-the sampled tokens on by itself, and the host's share of a step is hidden behind the GPU's.
+    plan    the scheduler says who runs and with how many tokens (`Scheduler.schedule`, or
+            `Scheduler.plan_ahead` for the step after one that is still on the GPU)
+    launch  the runner puts the pass and the sampling on the GPU and returns without waiting
+    retire  the tokens are read, the scheduler takes them in, and each goes to its request
 
-Clients on any thread talk to it through queues only: one inbox for submit and abort,
-one outbox per request that streams its tokens back.  It deals in token ids only.
+Up to two steps are under way: while the running requests do nothing but decode, the next
+step is planned and launched before this one is retired (the GPU hands the sampled tokens to
+it by itself), so the host's share of a step hides behind the GPU's.  A runner that has no
+`launch` (a fake in tests) is simply run in the launch stage.
+
+Clients on any thread reach the engine through one mailbox (requests and aborts) and get
+their tokens back through one stream per request; the engine's own state is touched by one
+thread only, the one that calls `step` (`start` makes a thread that does).  The engine deals
+in token ids only.  Public interface and meanings of the counters follow the reference
+(atomserve/engine.py:41-264).
 """
 
 import itertools
@@ -21,122 +26,156 @@ import sys
 import threading
 import time
 import traceback
-from dataclasses import dataclass
+from collections import deque
 from typing import Optional
 
 from atomserve_amd.cache.manager import CacheManager
 from atomserve_amd.config.engine_config import EngineConfig
 from atomserve_amd.engine.runner import ModelRunner
-from atomserve_amd.engine.scheduler import Scheduler, SchedulerOutput
+from atomserve_amd.engine.scheduler import Scheduler, StepPlan
 from atomserve_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus
 from atomserve_amd.kernels import ops
 
-
-@dataclass
-class _Finished:
-    reason: str  # "stop", "length", "abort" or "error"
-    error: Optional[BaseException] = None
+_END = object()  # last item of a request's stream
 
 
 class RequestHandle:
-    """The client's end of one request: iterate it to receive token ids as they are made;
-    afterwards `finish_reason` and the timing fields are set."""
+    """A client's view of its request: iterating yields the token ids as they are made and ends
+    when the request does; then `finish_reason` ("stop", "length", "abort" or "error") and the
+    timing fields are final.  A request that an engine failure ended raises RuntimeError."""
 
     def __init__(self, request_id: int, engine: "Engine", num_prompt_tokens: int):
         self.id = request_id
         self.num_prompt_tokens = num_prompt_tokens
         self.num_output_tokens = 0
-        self.num_cached_tokens = 0
+        self.num_cached_tokens = 0  # prompt tokens found in the prefix cache
         self.finish_reason: Optional[str] = None
         self.submitted_at = time.perf_counter()
         self.first_token_at: Optional[float] = None
         self.finished_at: Optional[float] = None
         self._engine = engine
-        self._outbox: queue.SimpleQueue = queue.SimpleQueue()
+        self._stream: queue.SimpleQueue = queue.SimpleQueue()  # lists of tokens, then (_END, reason, error)
 
     def __iter__(self):
         while True:
-            event = self._outbox.get()
-            if isinstance(event, _Finished):
-                self.finish_reason = event.reason
-                if event.error is not None:
-                    raise RuntimeError("engine step failed") from event.error
+            item = self._stream.get()
+            if isinstance(item, tuple) and item[0] is _END:
+                _, self.finish_reason, error = item
+                if error is not None:
+                    raise RuntimeError("engine step failed") from error
                 return
-            yield event
+            yield from item
 
     def abort(self) -> None:
         self._engine.abort(self.id)
 
     @property
-    def ttft(self):
-        """Seconds from submit to the first token."""
-        return None if self.first_token_at is None else self.first_token_at - self.submitted_at
+    def ttft(self) -> Optional[float]:
+        """Seconds between submission and the first token."""
+        if self.first_token_at is None:
+            return None
+        return self.first_token_at - self.submitted_at
 
     @property
-    def decode_tokens_per_s(self):
-        if self.first_token_at is None or self.finished_at is None or self.num_output_tokens < 2:
+    def decode_tokens_per_s(self) -> Optional[float]:
+        """Rate of the tokens after the first; None before the end or for replies of one token."""
+        if self.finished_at is None or self.first_token_at is None or self.num_output_tokens < 2:
             return None
         return (self.num_output_tokens - 1) / max(self.finished_at - self.first_token_at, 1e-9)
 
+    # engine side
+    def _deliver(self, tokens: list, now: float) -> None:
+        if self.first_token_at is None:
+            self.first_token_at = now
+        self.num_output_tokens += len(tokens)
+        self._stream.put(list(tokens))
+
+    def _end(self, seq: Sequence, error: Optional[BaseException]) -> None:
+        self.num_cached_tokens = seq.num_cached_tokens
+        self.finished_at = time.perf_counter()
+        self._stream.put((_END, seq.finish_reason or "error", error))
+
+
+class _Flight:
+    """A step between launch and retirement."""
+
+    __slots__ = ("plan", "pending")
+
+    def __init__(self, plan: StepPlan, pending):
+        self.plan, self.pending = plan, pending
+
+
+class _Ready:
+    """What a runner without `launch` leaves behind: results that are there already."""
+
+    device_tokens = None
+
+    def __init__(self, results):
+        self._results = results
+
+    def results(self):
+        return self._results
+
 
 class Engine:
+    MAX_IN_FLIGHT = 2
+
     def __init__(self, runner, scheduler: Scheduler, seed: Optional[int] = None):
         self.runner = runner
         self.scheduler = scheduler
-        self._inbox: queue.SimpleQueue = queue.SimpleQueue()
-        self._handles: dict = {}
-        self._ids = itertools.count()
+        self.run_ahead = True  # False: every step is retired before the next is planned
+        self._mail: queue.SimpleQueue = queue.SimpleQueue()  # ("submit", seq, handle) | ("abort", id) | ("wake",)
+        self._open: dict = {}  # request id -> handle, until the request ends
+        self._next_id = itertools.count()
+        self._seeds = random.Random(seed)  # for requests that bring no seed of their own
+        self._flights: deque = deque()
         self._thread: Optional[threading.Thread] = None
-        self._stopping = False
-        self._rng = random.Random(seed)  # seeds of the requests that bring none
-        self._in_flight = None  # (plan, pending step) of a decode step sent to the GPU ahead of its turn
-        self.run_ahead = True
-        self.num_steps = 0
-        self.last_batch_seqs = 0
-        self.last_batch_tokens = 0
-        self.num_prompt_tokens = 0
-        self.num_cached_prompt_tokens = 0
-        self.num_generated_tokens = 0
-        self.num_preemptions = 0
+        self._halt = threading.Event()
+        self.counters = dict.fromkeys(
+            ("steps", "last_batch_seqs", "last_batch_tokens", "prompt_tokens", "cached_prompt_tokens",
+             "generated_tokens", "preemptions"), 0)  # fmt: skip
 
-    # ---- client side (any thread) ---------------------------------------------------
+    # ---- clients (any thread) ---------------------------------------------------------------
     def submit(self, prompt_ids, params: SamplingParams) -> RequestHandle:
-        limit = self.scheduler.config.max_model_len
-        if not 0 < len(prompt_ids) < limit:
-            raise ValueError(f"prompt has {len(prompt_ids)} tokens; must be 1 to {limit - 1}")
+        ids = [int(t) for t in prompt_ids]
+        longest = self.scheduler.config.max_model_len
+        if not ids or len(ids) >= longest:
+            raise ValueError(f"prompt has {len(ids)} tokens; must be 1 to {longest - 1}")
         if params.max_tokens < 1:
             raise ValueError("max_tokens must be at least 1")
         vocab = getattr(self.runner, "vocab_size", None)
-        if vocab is not None and any(not 0 <= int(t) < vocab for t in prompt_ids):
+        if vocab is not None and (min(ids) < 0 or max(ids) >= vocab):
             raise ValueError(f"prompt holds a token id outside the vocabulary of {vocab}")
-        request_id = next(self._ids)
-        handle = RequestHandle(request_id, self, len(prompt_ids))
-        seq = Sequence(request_id, [int(t) for t in prompt_ids], params)
+        seq = Sequence(next(self._next_id), ids, params)
         if params.seed is None:
-            seq.noise_seed = self._rng.getrandbits(63)
-        self._inbox.put(("add", seq, handle))
+            seq.noise_seed = self._seeds.getrandbits(63)
+        handle = RequestHandle(seq.id, self, len(ids))
+        self._mail.put(("submit", seq, handle))
         return handle
 
     def abort(self, request_id: int) -> None:
-        self._inbox.put(("abort", request_id))
-
-    def start(self) -> None:
-        self._thread = threading.Thread(target=self._loop, name="atomserve-engine", daemon=True)
-        self._thread.start()
-
-    def shutdown(self) -> None:
-        self._stopping = True
-        self._inbox.put(("wake",))
-        if self._thread is not None:
-            self._thread.join()
+        self._mail.put(("abort", request_id))
 
     def generate(self, prompts, params: SamplingParams) -> list:
-        """Run prompts to completion on the calling thread; all are submitted first, so they
-        are batched together (reference atomserve/engine.py:137-146)."""
+        """Runs the prompts to their ends on the calling thread and returns their replies.  All are
+        submitted before the first step, so they share batches (reference atomserve/engine.py:137-146)."""
         handles = [self.submit(p, params) for p in prompts]
         while self.step():
             pass
         return [list(h) for h in handles]
+
+    def start(self) -> None:
+        """Serve on a thread of the engine's own until `shutdown`."""
+        self._halt.clear()
+        self._thread = threading.Thread(target=self._serve, name="atomserve-amd-engine", daemon=True)
+        self._thread.start()
+
+    def shutdown(self) -> None:
+        self._halt.set()
+        self._mail.put(("wake",))
+        if self._thread is not None:
+            self._thread.join()
+            self._thread = None
 
     def warm_up(self) -> int:
         """Before serving: the decode steps of every batch size up to max_num_seqs are captured now
@@ -148,132 +187,132 @@ class Engine:
         return graphs.capture_ahead(self.scheduler.config.max_num_seqs)
 
     def stats(self) -> dict:
-        s = self.scheduler
-        total = s.manager.num_blocks
-        used = total - s.manager.num_free
-        return {
-            "running": len(s.running),
-            "waiting": len(s.waiting),
+        manager = self.scheduler.manager
+        total = manager.num_blocks
+        used = total - manager.num_free
+        report = {
+            "running": len(self.scheduler.running),
+            "waiting": len(self.scheduler.waiting),
             "kv_blocks_used": used,
             "kv_blocks_total": total,
             "kv_usage": used / total,
-            "kv_blocks_cached": s.manager.num_cached,
-            "steps": self.num_steps,
-            "last_batch_seqs": self.last_batch_seqs,
-            "last_batch_tokens": self.last_batch_tokens,
-            "prompt_tokens": self.num_prompt_tokens,
-            "cached_prompt_tokens": self.num_cached_prompt_tokens,
-            "generated_tokens": self.num_generated_tokens,
-            "preemptions": self.num_preemptions,
+            "kv_blocks_cached": manager.num_cached,
         }
+        report.update(self.counters)
+        held = getattr(self.runner, "graph_bytes", None)
+        if held is not None:
+            report["graph_bytes"] = held()
+        return report
 
-    # ---- engine side (one thread) ---------------------------------------------------
+    @property
+    def steps_in_flight(self) -> int:
+        return len(self._flights)
+
+    # counters under the names they had as attributes
+    num_steps = property(lambda self: self.counters["steps"])
+    last_batch_seqs = property(lambda self: self.counters["last_batch_seqs"])
+    last_batch_tokens = property(lambda self: self.counters["last_batch_tokens"])
+    num_generated_tokens = property(lambda self: self.counters["generated_tokens"])
+    num_preemptions = property(lambda self: self.counters["preemptions"])
+
+    # ---- the pipeline (one thread) ----------------------------------------------------------
     def step(self) -> bool:
-        """One scheduling step; False when there is nothing to do."""
-        self._drain_inbox(block=False)
-        flight, self._in_flight = self._in_flight, None
-        if flight is not None:
-            out, pending = flight  # planned and sent to the GPU during the step before
-        else:
-            if not self.scheduler.has_work:
-                return False
-            out = self.scheduler.schedule()
-            if not out.seqs:
-                raise RuntimeError("scheduler has work but scheduled nothing")
-            launch = getattr(self.runner, "launch", None)
-            pending = launch(out) if launch is not None else None
-        sent = None
-        if pending is None:
-            results = self.runner.execute(out)
-        else:
-            ahead = self._plan_ahead(out)
-            if ahead is not None:
-                sent = (ahead, self.runner.launch(ahead, after=pending))
-            results = pending.results()
-        new_tokens = self.scheduler.update(out, results)
-        self._in_flight = sent  # only now: a step that failed on the way leaves nothing behind
-
-        now = time.perf_counter()
-        self.num_steps += 1
-        self.num_preemptions += len(out.preempted)
-        self.last_batch_seqs, self.last_batch_tokens = len(out.seqs), out.num_tokens
-        for seq, tokens in new_tokens:
-            handle = self._handles[seq.id]
-            if handle.first_token_at is None:
-                handle.first_token_at = now
-            handle.num_output_tokens += len(tokens)
-            self.num_generated_tokens += len(tokens)
-            for token in tokens:
-                handle._outbox.put(token)
-            if seq.status is SequenceStatus.FINISHED:
-                self._close(seq)
+        """Retires one step, launching what the pipeline needs before; False when there is nothing to
+        do.  If a stage raises, nothing stays in flight."""
+        self._read_mail(wait=False)
+        try:
+            if not self._flights:
+                if not self.scheduler.has_work:
+                    return False
+                plan = self.scheduler.schedule()
+                if not plan.seqs:
+                    raise RuntimeError("scheduler has work but scheduled nothing")
+                self._launch(plan, after=None)
+            if len(self._flights) < self.MAX_IN_FLIGHT:
+                self._launch_ahead(self._flights[-1])
+            self._retire(self._flights.popleft())
+        except BaseException:
+            self._flights.clear()
+            raise
         return True
 
-    def _plan_ahead(self, out):
-        """The decode step after `out`, if it is certain but for its tokens: `out` gives every running
-        request a token, nobody can be admitted or has left, nobody reaches its length with that token, no sampling
-        setting needs the tokens on the host, and every request has a page for one more position.  A
-        request that ends on an end-of-sequence token in `out` still takes part in the step ahead; its
-        result there is dropped and its pages, given back at once, may be written once more, which is
-        harmless: whoever gets them next writes after that, in the order of the GPU's queue."""
-        s = self.scheduler
-        can = getattr(self.runner, "can_run_ahead", None)
-        if not self.run_ahead or can is None or out.preempted or not self._inbox.empty():
-            return None
-        if s.waiting and len(s.running) < s.config.max_num_seqs:
-            return None  # somebody may be admitted next; with every place taken the queue just waits on
-        if len(out.seqs) != len(s.running) or any(a is not b for a, b in zip(out.seqs, s.running)):
-            return None
-        limit = s.config.max_model_len
-        for seq, n in zip(out.seqs, out.num_new_tokens):
-            p = seq.params
-            if (seq.status is not SequenceStatus.RUNNING or not seq.reaches_end(n) or p.presence_penalty != 0
-                    or seq.num_output_tokens + 1 >= p.max_tokens or seq.num_tokens + 1 >= limit):  # fmt: skip
-                return None
-        if not can(out.seqs):
-            return None
-        for seq in out.seqs:
-            if not s.manager.reserve(seq.cache, seq.num_tokens, 1):
-                return None  # the scheduler decides who makes room, in its own turn
-        return SchedulerOutput(seqs=list(out.seqs), num_new_tokens=[1] * len(out.seqs))
+    def _launch(self, plan: StepPlan, after) -> None:
+        launch = getattr(self.runner, "launch", None)
+        if launch is None:
+            pending = _Ready(self.runner.execute(plan))
+        else:
+            pending = launch(plan, after=after.pending if after is not None else None)
+        self._flights.append(_Flight(plan, pending))
 
-    def _drain_inbox(self, block: bool) -> None:
+    def _launch_ahead(self, head: _Flight) -> None:
+        """Plans and launches the decode step after `head` if it is certain already: the scheduler says
+        so, no message waits that could change who runs, no request needs its tokens on the host
+        before the next sampling (a presence penalty does), and the runner can feed a step from the
+        GPU's own tokens."""
+        can = getattr(self.runner, "can_run_ahead", None)
+        if not self.run_ahead or can is None or not self._mail.empty():
+            return
+        if any(seq.params.presence_penalty != 0 for seq in head.plan.seqs) or not can(head.plan.seqs):
+            return
+        plan = self.scheduler.plan_ahead(head.plan)
+        if plan is not None:
+            self._launch(plan, after=head)
+
+    def _retire(self, flight: _Flight) -> None:
+        results = flight.pending.results()
+        gained = self.scheduler.update(flight.plan, results)
+        now = time.perf_counter()
+        c = self.counters
+        c["steps"] += 1
+        c["preemptions"] += len(flight.plan.preempted)
+        c["last_batch_seqs"], c["last_batch_tokens"] = len(flight.plan.seqs), flight.plan.num_tokens
+        for seq, tokens in gained:
+            c["generated_tokens"] += len(tokens)
+            self._open[seq.id]._deliver(tokens, now)
+            if seq.status is SequenceStatus.FINISHED:
+                self._close(seq)
+
+    def _close(self, seq: Sequence, error: Optional[BaseException] = None) -> None:
+        handle = self._open.pop(seq.id)
+        self.counters["cached_prompt_tokens"] += seq.num_cached_tokens
+        self.runner.sampler.release(seq.id)
+        handle._end(seq, error)
+
+    def _read_mail(self, wait: bool) -> None:
+        """Takes in every message that is there; with `wait`, sleeps until there is one."""
         while True:
             try:
-                message = self._inbox.get(block=block)
+                message = self._mail.get(block=wait)
             except queue.Empty:
                 return
-            block = False
-            if message[0] == "add":
+            wait = False
+            kind = message[0]
+            if kind == "submit":
                 _, seq, handle = message
-                self._handles[seq.id] = handle
-                self.num_prompt_tokens += seq.num_prompt_tokens
+                self._open[seq.id] = handle
+                self.counters["prompt_tokens"] += seq.num_prompt_tokens
                 self.scheduler.add(seq)
-            elif message[0] == "abort":
+            elif kind == "abort":
                 seq = self.scheduler.abort(message[1])
                 if seq is not None:
                     self._close(seq)
 
-    def _close(self, seq: Sequence, error: Optional[BaseException] = None) -> None:
-        handle = self._handles.pop(seq.id)
-        handle.num_cached_tokens = seq.num_cached_tokens
-        self.num_cached_prompt_tokens += seq.num_cached_tokens
-        handle.finished_at = time.perf_counter()
-        self.runner.sampler.release(seq.id)
-        handle._outbox.put(_Finished(seq.finish_reason or "error", error))
-
-    def _loop(self) -> None:
-        while not self._stopping:
+    def _serve(self) -> None:
+        while not self._halt.is_set():
             try:
                 if not self.step():
-                    self._drain_inbox(block=True)
-            except Exception as error:  # fail the requests, keep the engine alive
+                    self._read_mail(wait=True)
+            except Exception as error:
+                # the requests that were under way fail with the error; the thread goes on serving
                 traceback.print_exc(file=sys.stderr)
-                self._in_flight = None
-                for seq in [*self.scheduler.running, *self.scheduler.waiting]:
-                    self.scheduler.abort(seq.id)
-                    seq.finish_reason = "error"
-                    self._close(seq, error)
+                self._fail_all(error)
+
+    def _fail_all(self, error: BaseException) -> None:
+        self._flights.clear()
+        for seq in list(self.scheduler.running) + list(self.scheduler.waiting):
+            self.scheduler.abort(seq.id)
+            seq.finish_reason = "error"
+            self._close(seq, error)
 
 
 def create_engine(model, engine_config: EngineConfig, eos_token_ids=frozenset(), seed: Optional[int] = None) -> Engine:

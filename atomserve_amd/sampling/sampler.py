@@ -67,24 +67,29 @@ class Sampler:
         return out
 
     def _apply_presence_penalty(self, logits, seqs):
-        """Subtract each row's penalty from the logits of the tokens it has generated so far
-        (reference atomserve/sampler.py:144-168)."""
-        rows, cols, amounts = [], [], []
-        for i, seq in enumerate(seqs):
-            if seq.params.presence_penalty != 0:
-                seen = set(seq.output_ids)
-                rows.extend([i] * len(seen))
-                cols.extend(seen)
-                amounts.extend([seq.params.presence_penalty] * len(seen))
-        if not rows:
+        """logits with each penalised row's amount taken off every token the row's request has
+        generated so far, each token once however often it came (reference atomserve/sampler.py:144-168).
+        The rows are copied first: the caller's logits stay as the model made them."""
+        marks = []  # per penalised row: (row, its distinct generated tokens, amount)
+        for row, seq in enumerate(seqs):
+            amount = seq.params.presence_penalty
+            if amount != 0 and seq.num_output_tokens:
+                marks.append((row, np.unique(np.asarray(seq.output_ids, dtype=np.int32)), amount))
+        if not marks:
             return logits
+        total = sum(len(tokens) for _, tokens, _ in marks)
+        # one upload: [rows | tokens | amounts as bit patterns]
+        host = np.empty(3 * total, dtype=np.int32)
+        at = 0
+        for row, tokens, amount in marks:
+            n = len(tokens)
+            host[at : at + n] = row
+            host[total + at : total + at + n] = tokens
+            host[2 * total + at : 2 * total + at + n].view(np.float32)[:] = amount
+            at += n
+        dev = torch.from_numpy(host).to(self.device, non_blocking=True)
         logits = logits.clone()
-        ops.apply_penalty(
-            logits,
-            torch.tensor(rows, dtype=torch.int32).to(self.device),
-            torch.tensor(cols, dtype=torch.int32).to(self.device),
-            torch.tensor(amounts, dtype=torch.float32).to(self.device),
-        )
+        ops.apply_penalty(logits, dev[:total], dev[total : 2 * total], dev[2 * total :].view(torch.float32))
         return logits
 
 

@@ -122,7 +122,7 @@ def test_requests_without_a_seed_get_distinct_streams_and_seeded_ones_keep_their
     e.submit([1], SamplingParams())
     e.submit([1], SamplingParams())
     e.submit([1], SamplingParams(seed=42))
-    e._drain_inbox(block=False)
+    e._read_mail(wait=False)
     a, b, c = e.scheduler.waiting
     assert a.noise_seed != b.noise_seed and c.noise_seed == 42
 
@@ -183,7 +183,7 @@ def test_steps_sent_ahead_change_nothing_but_the_time(eos):
                 late = e.submit([3, 1, 4, 1, 5], params[0])  # arrives while others decode
         handles.append(late)
         outs = [(list(h), h.finish_reason) for h in handles]
-        assert e.stats()["kv_blocks_used"] == 0 and e._in_flight is None
+        assert e.stats()["kv_blocks_used"] == 0 and e.steps_in_flight == 0
         return outs
 
     plain = run(CountingRunner())
@@ -220,4 +220,4 @@ def test_a_failing_step_leaves_no_step_behind_it():
     alone = engine().generate([[4, 5]], GREEDY)[0]
     assert list(e.submit([4, 5], GREEDY)) == alone
     e.shutdown()
-    assert e._in_flight is None and e.stats()["kv_blocks_used"] == 0 and e.runner.sent_ahead > 2
+    assert e.steps_in_flight == 0 and e.stats()["kv_blocks_used"] == 0 and e.runner.sent_ahead > 2
