@@ -14,6 +14,7 @@
 // through LDS, partitions by attn_reduce.  Serves fp32 (every row) and bf16 (decode).
 // Plain reference: reference atomserve/kernels.py:167-334, atomserve/model.py:269-289.
 #include "common.h"
+#include "no_alloc.h"
 #include <type_traits>
 
 #define NEG_INF (-__builtin_inff())
@@ -1070,4 +1071,49 @@ extern "C" int as_attn_single_query(const void* q, const void* k_pages, const vo
                                      table_width, out, part_m, part_l, part_acc, H, KV, D, bs, scale, window,
                                      part_size, P, stream);
   return AS_BAD_DTYPE;
+}
+
+// ---- the same without scratch buffers from the caller ----------------------------------
+//
+// The partial results of a split context live in an array of the library's own; see no_alloc.h.
+// In host code `scratch` is only a stand-in for the symbol: the address that kernels and copies
+// use is the one hipGetSymbolAddress returns, and every GPU has its own.
+static __device__ __align__(256) float scratch[AS_STATIC_SCRATCH_FLOATS];
+static float* scratch_on_device[64] = {nullptr};
+
+static int scratch_of_current_device(float** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return AS_LAUNCH_FAILED;
+  if (scratch_on_device[dev] == nullptr) {
+    void* found = nullptr;
+    if (hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)) != hipSuccess || found == nullptr) return AS_LAUNCH_FAILED;
+    scratch_on_device[dev] = (float*)found;
+  }
+  *ptr = scratch_on_device[dev];
+  return AS_OK;
+}
+
+extern "C" int as_attn_single_query_static(const void* q, const void* k_pages, const void* v_pages, int dtype,
+                                           const int* items, int num_items, const int* positions,
+                                           const int* tok_row, const int* block_tables, int table_width,
+                                           void* out, int H, int KV, int D, int bs, float scale, int window,
+                                           int part_size, int P, hipStream_t stream) {
+  if (num_items <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || H % KV || D <= 0 || bs <= 0 || part_size <= 0 || P <= 0 || table_width <= 0)
+    return AS_BAD_SHAPE;
+  float *part_m = nullptr, *part_l = nullptr, *part_acc = nullptr;
+  if (P > 1) {
+    const unsigned long long rows = (unsigned long long)num_items * (unsigned long long)H * (unsigned long long)P;
+    if (rows > AS_STATIC_SCRATCH_FLOATS || rows * (unsigned long long)(D + 2) > AS_STATIC_SCRATCH_FLOATS)
+      return AS_TOO_LARGE;
+    float* base = nullptr;
+    const int status = scratch_of_current_device(&base);
+    if (status != AS_OK) return status;
+    part_acc = base;  // [rows, D]: first, so that it keeps the array's alignment
+    part_m = base + rows * D;
+    part_l = part_m + rows;
+  }
+  return as_attn_single_query(q, k_pages, v_pages, dtype, items, num_items, positions, tok_row, block_tables,
+                              table_width, out, part_m, part_l, part_acc, H, KV, D, bs, scale, window,
+                              part_size, P, stream);
 }

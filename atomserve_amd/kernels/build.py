@@ -20,7 +20,7 @@ ARCH = "gfx950"
 # Packed fp32 instructions are switched off for every kernel of this package.
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]  # fmt: skip
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 LIBRARIES = ("elementwise", "attention", "gemm", "sampling", "blas")
 LINK = {"blas": ["-lhipblaslt"]}  # what a library links beside the HIP runtime
 

@@ -40,7 +40,8 @@ SIGNATURES = {
     "as_topk": ("sampling", [P, I, I, I, P, P, P]),
 }
 
-STATUS = {-1: "unsupported dtype", -2: "unsupported shape or size", -3: "kernel launch failed"}
+STATUS = {-1: "unsupported dtype", -2: "unsupported shape or size", -3: "kernel launch failed",
+          -4: "partial results exceed the library's static scratch array"}
 
 _libs: dict = {}
 _funcs: dict = {}
