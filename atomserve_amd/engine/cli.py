@@ -20,6 +20,52 @@ from atomserve_amd import __version__
 DTYPES = ("bf16", "fp32")
 
 
+def kv_budget(text: str):
+    """--kv-mem-gb: a number of GiB, or 'auto'."""
+    if text.strip().lower() == "auto":
+        return "auto"
+    try:
+        value = float(text)
+    except ValueError:
+        raise argparse.ArgumentTypeError(f"{text!r} is neither a number of GiB nor 'auto'") from None
+    if value <= 0:
+        raise argparse.ArgumentTypeError("the KV cache needs a positive amount of memory")
+    return value
+
+
+def fit_kv_budget(wanted, free_bytes: int, reserve_bytes: int, note=print) -> float:
+    """The GiB the cache pool gets: what was asked for, cut down to what the GPU has free after
+    the weights minus a reserve for a step's activations, its logits and the libraries' workspaces
+    (the reference shrinks its budget the same way on its device, atomserve/cli.py:122-136).
+    'auto' takes all of that room.  Exits with a message when no room worth a pool is left."""
+    room = (free_bytes - reserve_bytes) / 2**30
+    if room < 0.25:
+        raise SystemExit(
+            f"atomserve: the weights leave {free_bytes / 2**30:.1f} GiB of GPU memory free, of which "
+            f"{reserve_bytes / 2**30:.1f} GiB are kept for activations: no room for a KV cache "
+            "(a smaller model, or --dtype bf16, leaves more)"
+        )
+    if wanted == "auto":
+        return room
+    if wanted > room:
+        note(f"Note: KV cache reduced from {wanted:.1f} to {room:.1f} GiB to fit in GPU memory.")
+        return room
+    return float(wanted)
+
+
+def step_reserve_bytes(plan, max_batched_tokens: int, max_num_seqs: int) -> int:
+    """Memory a step needs beside weights and cache, generously: the rows of a full step in every
+    width a layer makes of them, the logits of the replayed decode steps, and the libraries."""
+    widest = 0
+    for layer in plan.layers:
+        mixer, ffn = layer.mixer, layer.ffn
+        heads = getattr(mixer, "num_heads", 0) + 2 * getattr(mixer, "num_kv_heads", 0)
+        widest = max(widest, 8 * plan.hidden_size + 8 * heads * getattr(mixer, "head_dim", 0)
+                     + 12 * getattr(ffn, "intermediate_size", plan.hidden_size))  # fmt: skip
+    logits = 4 * plan.vocab_size * (2 * min(256, max_num_seqs) + 64)
+    return (1 << 30) + 2 * max_batched_tokens * widest + logits
+
+
 def build_parser() -> argparse.ArgumentParser:
     p = argparse.ArgumentParser(
         prog="atomserve",
@@ -29,7 +75,9 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("model", help="local model directory (config.json + *.safetensors); with --random-weights, "
                                  "a directory or file holding only config.json")  # fmt: skip
     p.add_argument("--dtype", choices=DTYPES, default="bf16", help="weights, activations and the KV cache")
-    p.add_argument("--kv-mem-gb", type=float, default=4.0, help="GiB of memory for the KV cache")
+    p.add_argument("--kv-mem-gb", type=kv_budget, default=4.0,
+                   help="GiB of memory for the KV cache, or 'auto' for all that the weights leave free; "
+                        "reduced with a note if the GPU has less left")  # fmt: skip
     p.add_argument("--block-size", type=int, default=16, help="tokens per KV block")
     p.add_argument("--max-num-seqs", type=int, default=32, help="most requests running at once")
     p.add_argument("--max-batched-tokens", type=int, default=512,
@@ -59,6 +107,8 @@ def engine_config_for(args, bytes_per_block: int, max_positions: int):
     (reference atomserve/cli.py:99-119)."""
     from atomserve_amd.config import EngineConfig
 
+    if args.kv_mem_gb == "auto":
+        raise ValueError("the budget must be fitted to the GPU first (fit_kv_budget)")
     num_blocks = int(args.kv_mem_gb * 2**30 // bytes_per_block)
     if num_blocks < 1:
         raise SystemExit("atomserve: --kv-mem-gb leaves no room for a single KV block")
@@ -125,6 +175,14 @@ def main(argv=None) -> int:
     else:
         load_weights(model_dir, model, arch, config)
     block_bytes = CachePools.bytes_per_block(model.cache_requests(), args.block_size, dtype) or 1
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()  # what loading used for conversions counts as free
+    free_bytes, _ = torch.cuda.mem_get_info()
+    args.kv_mem_gb = fit_kv_budget(args.kv_mem_gb, free_bytes,
+                                   step_reserve_bytes(model.plan, args.max_batched_tokens, args.max_num_seqs),
+                                   note=lambda text: print(text, file=sys.stderr, flush=True))  # fmt: skip
+    if args.kv_mem_gb * 2**30 // block_bytes > 2**31 // args.block_size:  # slots are 32-bit integers
+        args.kv_mem_gb = (2**31 // args.block_size) * block_bytes / 2**30
     engine_config = engine_config_for(args, block_bytes, model.plan.max_positions)
     engine = create_engine(model, engine_config, eos_ids(model_dir), seed=args.seed)
     engine.generate([[0]], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))  # compile and warm up

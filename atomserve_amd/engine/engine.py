@@ -131,6 +131,7 @@ class Engine:
         self._flights: deque = deque()
         self._thread: Optional[threading.Thread] = None
         self._halt = threading.Event()
+        self._phases = None
         self.counters = dict.fromkeys(
             ("steps", "last_batch_seqs", "last_batch_tokens", "prompt_tokens", "cached_prompt_tokens",
              "generated_tokens", "preemptions"), 0)  # fmt: skip
@@ -186,6 +187,17 @@ class Engine:
             return 0
         return graphs.capture_ahead(self.scheduler.config.max_num_seqs)
 
+    def profile_phases(self, on: bool = True):
+        """Starts (or ends) the split of the host's time by phase; returns the `PhaseTimes` that
+        collects it.  While it is on no step is launched ahead, so that the wait for the GPU shows
+        as what it is."""
+        from atomserve_amd.engine.runner import PhaseTimes
+
+        self._phases = PhaseTimes() if on else None
+        if hasattr(self.runner, "phases"):
+            self.runner.phases = self._phases
+        return self._phases
+
     def stats(self) -> dict:
         manager = self.scheduler.manager
         total = manager.num_blocks
@@ -220,17 +232,25 @@ class Engine:
         """Retires one step, launching what the pipeline needs before; False when there is nothing to
         do.  If a stage raises, nothing stays in flight."""
         self._read_mail(wait=False)
+        phases = self._phases
         try:
             if not self._flights:
                 if not self.scheduler.has_work:
                     return False
+                if phases is not None:
+                    phases.begin()
                 plan = self.scheduler.schedule()
                 if not plan.seqs:
                     raise RuntimeError("scheduler has work but scheduled nothing")
+                if phases is not None:
+                    phases.mark("schedule")
                 self._launch(plan, after=None)
-            if len(self._flights) < self.MAX_IN_FLIGHT:
+            if len(self._flights) < self.MAX_IN_FLIGHT and phases is None:
                 self._launch_ahead(self._flights[-1])
             self._retire(self._flights.popleft())
+            if phases is not None:
+                phases.mark("update")
+                phases.steps += 1
         except BaseException:
             self._flights.clear()
             raise

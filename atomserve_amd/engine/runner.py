@@ -33,6 +33,35 @@ def rows_for(seqs, num_new_tokens) -> list:
     return rows
 
 
+class PhaseTimes:
+    """Where the host's time of a step goes: seconds per phase, summed over steps.  The engine and the
+    runner call `mark(phase)` at the end of each phase when one of these is installed
+    (`Engine.profile_phases`); the phases are those of the reference's bench/engine.py:129-171:
+    schedule, pack (rows, flat integers, upload), launch (the pass put on the GPU), sample (the
+    sampling kernels put on the GPU), wait (for the GPU), update (tokens taken in and handed out)."""
+
+    PHASES = ("schedule", "pack", "launch", "sample", "wait", "update")
+
+    def __init__(self):
+        import time
+
+        self._now = time.perf_counter
+        self.seconds = dict.fromkeys(self.PHASES, 0.0)
+        self.steps = 0
+        self._last = self._now()
+
+    def begin(self) -> None:
+        self._last = self._now()
+
+    def mark(self, phase: str) -> None:
+        now = self._now()
+        self.seconds[phase] += now - self._last
+        self._last = now
+
+    def mean_us(self) -> dict:
+        return {k: round(v / max(1, self.steps) * 1e6, 1) for k, v in self.seconds.items()}
+
+
 def _bucket(n: int, steps) -> int:
     for s in steps:
         if n <= s:
@@ -132,6 +161,8 @@ class DecodeGraphs:
             if tokens_from is not None:
                 entry[1].token_ids[: len(rows)].copy_(tokens_from)
         graph, batch, logits = entry
+        if r.phases is not None:
+            r.phases.mark("pack")
         graph.replay()
         wanted = [i for i, row in enumerate(rows) if row.want]
         if wanted == list(range(len(rows))):
@@ -157,7 +188,8 @@ class DecodeGraphs:
 class PendingStep:
     """A step that is on the GPU, sampling included; `results()` waits for its tokens."""
 
-    def __init__(self, samples, num_computed, device_tokens, host_tokens, event):
+    def __init__(self, samples, num_computed, device_tokens, host_tokens, event, phases=None):
+        self.phases = phases
         self.samples = samples  # per scheduled sequence: whether the step gives it a token
         self.num_computed = num_computed  # per scheduled sequence: its leading tokens in the cache afterwards
         self.device_tokens = device_tokens  # int32 on the GPU, one per sampling sequence, or None
@@ -168,6 +200,8 @@ class PendingStep:
         tokens = iter(())
         if self.device_tokens is not None:
             self.event.synchronize()
+            if self.phases is not None:
+                self.phases.mark("wait")
             tokens = iter(self.host_tokens[: self.device_tokens.shape[0]].tolist())
         return [StepResult([next(tokens)] if yes else [], n) for yes, n in zip(self.samples, self.num_computed)]
 
@@ -186,6 +220,7 @@ class ModelRunner:
         self.decode_graphs = DecodeGraphs(self) if use_graphs else None
         self._token_buffers = []  # pinned, used in turn: the sampled tokens of the steps on their way
         self._token_turn = 0
+        self.phases = None  # a PhaseTimes while the host's time is being split up
 
     def prepare(self, rows, **layout) -> StepBatch:
         return StepBatch(rows, self.manager.block_size, len(self.manager.paged_groups), self.vocab_size,
@@ -202,6 +237,8 @@ class ModelRunner:
         if tokens_from is not None:
             raise ValueError("only a replayed decode step takes its tokens from the GPU")
         batch = self.prepare(rows)
+        if self.phases is not None:
+            self.phases.mark("pack")
         return self.model.forward(batch)
 
     @torch.inference_mode()
@@ -237,6 +274,8 @@ class ModelRunner:
             num_computed = [s.num_tokens + 1 for s in out.seqs]
             rows = [Row([0], s.num_tokens, s.cache.tables, [0], s.cache.state_slot) for s in out.seqs]
             logits = self.step(rows, tokens_from=after.device_tokens)
+        if self.phases is not None:
+            self.phases.mark("launch")
         sampling = [s for s, yes in zip(out.seqs, samples) if yes]
         device_tokens = self.sampler.launch(logits, sampling, ahead=0 if after is None else 1)
         host_tokens = event = None
@@ -252,4 +291,6 @@ class ModelRunner:
             host_tokens[: device_tokens.shape[0]].copy_(device_tokens, non_blocking=True)
             event = torch.cuda.Event()
             event.record()
-        return PendingStep(samples, num_computed, device_tokens, host_tokens, event)
+        if self.phases is not None:
+            self.phases.mark("sample")
+        return PendingStep(samples, num_computed, device_tokens, host_tokens, event, self.phases)

@@ -40,7 +40,7 @@ SIZES = {
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=128)
+    p.add_argument("--steps", type=int, default=256, help="decode steps timed: every sequence generates this many tokens")
     p.add_argument("--warmup", type=int, default=8)
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=2048)
@@ -60,6 +60,10 @@ def parse_args():
                         "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
                         "scheduler from submission to the last token")  # fmt: skip
     p.add_argument("--chunk-budget", type=int, default=512, help="token budget of a step in the mixed workload")
+    p.add_argument("--profile", action="store_true",
+                   help="also split the host's time of a decode step into schedule / pack / launch / sample / wait / "
+                        "update (steps run one at a time meanwhile, none sent ahead), as the reference's "
+                        "bench/engine.py --profile does")  # fmt: skip
     return p.parse_args()
 
 
@@ -190,7 +194,8 @@ def main() -> int:
 
     batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
     block = args.block_size
-    max_len = max(args.max_len, args.context + args.steps + args.warmup + 16, args.prefill_tokens + 16)
+    max_len = max(args.max_len, args.context + args.steps + args.warmup + 16 + (64 if args.profile else 0),
+                  args.prefill_tokens + 16)
     num_blocks = max(batches) * max_len // block
     params = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True) if args.greedy else \
         SamplingParams(max_tokens=100000, ignore_eos=True)  # fmt: skip
@@ -206,7 +211,16 @@ def main() -> int:
     weight_bytes = (layer_params * c.num_layers + c.vocab_size * c.hidden_size) * itemsize
     kv_bytes_per_token = c.num_layers * 2 * c.num_kv_heads * c.head_dim * itemsize
 
-    def run_decode(batch: int, steps: int, warmup: int):
+    host_phases = {}
+
+    def roofline(batch: int, mean_ctx: float, ms: float) -> dict:
+        """The bytes a decode step has to read (every weight once, the cache of the live requests)
+        over its time, against the HBM peak."""
+        achieved = (weight_bytes + batch * mean_ctx * kv_bytes_per_token) / (ms * 1e-3)
+        return {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK, 4)}  # fmt: skip
+
+    def run_decode(batch: int, steps: int, warmup: int, profile: int = 0):
         """Prefill `batch` prompts of args.context tokens (untimed), then time `steps` decode steps."""
         handles = [engine.submit(prompt(b, args.context, c.vocab_size), params) for b in range(batch)]
         while any(s.num_computed_tokens < s.num_prompt_tokens for s in
@@ -223,6 +237,12 @@ def main() -> int:
         dt = time.perf_counter() - t0
         assert len(engine.scheduler.running) == batch and engine.last_batch_tokens == batch
         mean_ctx = ctx_start + steps / 2
+        if profile:
+            phases = engine.profile_phases(True)
+            for _ in range(profile):
+                engine.step()
+            engine.profile_phases(False)
+            host_phases.update(phases.mean_us())
         for h in handles:
             engine.abort(h.id)
         engine.step()
@@ -248,14 +268,13 @@ def main() -> int:
         result_prefill = {"value": round(T / dt, 1), "tokens": T, "ms": round(dt * 1e3, 3),
                           "frac": round(flops / dt / PEAK_FLOPS[args.dtype], 4)}  # fmt: skip
 
-    points = {}
+    points, point_rooflines = {}, {}
     for b in batches:
         if b != args.batch:
-            tps, ms, _ = run_decode(b, max(16, args.steps // 4), max(2, args.warmup // 2))
+            tps, ms, ctx = run_decode(b, max(16, args.steps // 4), max(2, args.warmup // 2))
             points[f"decode_b{b}"] = round(tps, 1)
-    tps, ms, mean_ctx = run_decode(args.batch, args.steps, args.warmup)
-    step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
-    achieved = step_bytes / (ms * 1e-3)
+            point_rooflines[f"decode_b{b}"] = roofline(b, ctx, ms)
+    tps, ms, mean_ctx = run_decode(args.batch, args.steps, args.warmup, profile=64 if args.profile else 0)
 
     line = {
         "metric": f"decode tok/s at batch {args.batch}, {args.context}-token contexts (Qwen3-{args.sizes.upper()} sizes, random weights)",
@@ -277,10 +296,14 @@ def main() -> int:
             "seq_len": args.context, "max_context": max_len, "block_size": block, "parallelism": "single GPU",
             "sampling": "greedy" if args.greedy else "temperature 0.6 top-k 20 top-p 0.95",
         },
-        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4)},  # fmt: skip
+        "roofline": roofline(args.batch, mean_ctx, ms),
         "points": points,
+        "roofline_points": point_rooflines,
     }
+    if host_phases:
+        line["host_phases_us"] = host_phases
+        print("host time of a decode step without steps sent ahead, microseconds: "
+              + ", ".join(f"{k} {v}" for k, v in host_phases.items()), file=sys.stderr)  # fmt: skip
     if result_prefill:
         line["prefill"] = result_prefill
     if calibration:

@@ -50,3 +50,33 @@ def test_bytes_per_block_of_a_model():
 
 def test_prompt_ids_are_parsed():
     assert parse_ids("1, 2,3  4") == [1, 2, 3, 4]
+
+
+def test_the_budget_is_fitted_to_what_the_gpu_has_left():
+    """reference atomserve/cli.py:122-136: the budget shrinks to the room, with a note; no room is an error."""
+    from atomserve_amd.engine.cli import fit_kv_budget, kv_budget
+
+    gib = 2**30
+    notes = []
+    assert fit_kv_budget(4.0, 100 * gib, 2 * gib, notes.append) == 4.0 and not notes
+    assert fit_kv_budget(4.0, 5 * gib, 2 * gib, notes.append) == 3.0 and "reduced from 4.0 to 3.0" in notes[0]
+    assert fit_kv_budget("auto", 100 * gib, 2 * gib, notes.append) == 98.0 and len(notes) == 1
+    with pytest.raises(SystemExit, match="no room for a KV cache"):
+        fit_kv_budget(4.0, 2 * gib, 2 * gib, notes.append)
+    assert kv_budget("auto") == "auto" and kv_budget("2.5") == 2.5
+    assert build_parser().parse_args(["m", "--kv-mem-gb", "auto"]).kv_mem_gb == "auto"
+    with pytest.raises(SystemExit):
+        build_parser().parse_args(["m", "--kv-mem-gb", "-1"])
+
+
+def test_the_reserve_of_a_step_grows_with_its_budget_and_the_vocabulary():
+    from atomserve_amd.config.model_config import Qwen3Config
+    from atomserve_amd.engine.cli import step_reserve_bytes
+    from atomserve_amd.models.qwen3 import build_plan
+
+    cfg = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_layers=2, num_heads=32, num_kv_heads=8,
+               head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False, max_position_embeddings=4096)  # fmt: skip
+    plan = build_plan(Qwen3Config(**cfg))
+    small, large = step_reserve_bytes(plan, 512, 32), step_reserve_bytes(plan, 8192, 32)
+    assert 2**30 < small < large < 8 * 2**30
+    assert step_reserve_bytes(build_plan(Qwen3Config(**{**cfg, "vocab_size": 1000})), 512, 32) < small
