@@ -5,7 +5,8 @@ in the compute dtype: the block_size keys of one head in one page are contiguous
 the value half of a page is stored transposed, [D, block_size].  It
 starts zeroed, so that no slot ever holds a non-finite value
 (reference atomserve/kv_cache.py:112-118).  A state group has
-[caches in group, max_num_seqs, *shape].
+[caches in group, max_num_seqs + 1, *shape]: one slot per running request and a last one
+(`scrap_slot`) that belongs to nobody, for the rows that only pad a captured step.
 """
 
 import torch
@@ -23,8 +24,9 @@ class CachePools:
             shape = (len(g.cache_ids), 2, manager.num_blocks, r.num_kv_heads, manager.block_size, r.head_dim)
             self.paged.append(torch.zeros(shape, dtype=dtype, device=device))
         self.state = []
+        self.scrap_slot = manager.max_num_seqs
         for g in manager.state_groups:
-            shape = (len(g.cache_ids), manager.max_num_seqs, *g.request.shape)
+            shape = (len(g.cache_ids), manager.max_num_seqs + 1, *g.request.shape)
             self.state.append(torch.zeros(shape, dtype=g.request.dtype, device=device))
 
     def pages(self, cache_id: int):
@@ -39,7 +41,7 @@ class CachePools:
         return gi, k, self.paged[gi][li, 1].view(nb, kv, d, bs)
 
     def state_of(self, cache_id: int):
-        """(group index, state tensor [max_num_seqs, *shape]) of one cache."""
+        """(group index, state tensor [max_num_seqs + 1, *shape]) of one cache."""
         kind, gi, li = self.manager.group_of_cache[cache_id]
         if kind != "state":
             raise KeyError(f"cache {cache_id} holds no fixed-size state")

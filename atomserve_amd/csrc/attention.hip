@@ -450,7 +450,8 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
           const int i = lane + p * WAVE;
           if (i < HALF) {
             const float a = (float)ka[p] * kinv * gka[p], b = (float)kb2[p] * kinv * gkb[p];
-            const bf16 ra = (bf16)(a * kcs[p].x - b * kcs[p].y), rb = (bf16)(b * kcs[p].x + a * kcs[p].y);
+            const bf16 ra = finite_or_zero((bf16)(a * kcs[p].x - b * kcs[p].y));
+            const bf16 rb = finite_or_zero((bf16)(b * kcs[p].x + a * kcs[p].y));
             fresh_kv[0][i] = ra;
             fresh_kv[0][i + HALF] = rb;
             if (slot >= 0) { dst[i] = ra; dst[i + HALF] = rb; }
@@ -462,8 +463,9 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         for (int p = 0; p < 2 * PAIRS; ++p) {
           const int i = lane + p * WAVE;
           if (i < D) {
-            fresh_kv[1][i] = vv[p];
-            if (slot >= 0) vt[(size_t)i * bs] = vv[p];
+            const bf16 rv = finite_or_zero((bf16)vv[p]);
+            fresh_kv[1][i] = rv;
+            if (slot >= 0) vt[(size_t)i * bs] = rv;
           }
         }
       }
@@ -938,6 +940,7 @@ static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_
   if (fresh && D % 64) return AS_BAD_SHAPE;
   dim3 grid(num_items, KV, P);
   const size_t shmem = sizeof(float) * (size_t)(128 + 4 * D * G);
+  if (shmem + 1024 > (64u << 10)) return AS_BAD_SHAPE;  // wide heads in large groups: the general kernel's
   const FreshQKV none = {};
 #define LAUNCH(DCV, FRESHV)                                                                               \
   attn_decode_mfma_kernel<DCV, FRESHV><<<grid, 256, shmem, stream>>>(                                     \

@@ -25,6 +25,16 @@ template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return (bf16)v; }  // round to nearest even
 
+// What the cache pools may hold: a value that is not finite (a model that overflowed) is stored
+// as zero.  Kernels multiply keys and values of masked places by a weight of zero, which is only
+// harmless while every stored value is finite; pages are used again by other requests.
+__device__ __forceinline__ float finite_or_zero(float v) {
+  return (__float_as_uint(v) & 0x7f800000u) == 0x7f800000u ? 0.f : v;
+}
+__device__ __forceinline__ bf16 finite_or_zero(bf16 v) {
+  return (__builtin_bit_cast(unsigned short, v) & 0x7f80u) == 0x7f80u ? (bf16)0.f : v;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);

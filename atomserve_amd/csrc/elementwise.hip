@@ -4,30 +4,51 @@
 #include "common.h"
 
 // ---- embedding --------------------------------------------------------------------
-// out[t, :] = table[ids[t], :] as fp32 (the residual stream is always fp32).
+// out[t, :] = scale * table[ids[t], :] as fp32 (the residual stream is always fp32; the scale is 1
+// for models that do not multiply their embeddings).
 // Plain reference: reference atomserve/model.py:373.
 template <typename T>
 __global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ out, int width, int vocab) {
+                                    float* __restrict__ out, int width, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // ids are validated on the host; never read outside
   const T* src = table + (size_t)id * width;
   float* dst = out + (size_t)t * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_f32(src[i]);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_f32(src[i]) * scale;
 }
 
 extern "C" int as_embed_gather(const void* table, int table_dtype, const int* ids, float* out,
-                               int num_tokens, int width, int vocab, hipStream_t stream) {
+                               int num_tokens, int width, int vocab, float scale, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
   if (width <= 0 || vocab <= 0) return AS_BAD_SHAPE;
   const int threads = width >= 1024 ? 256 : 64;
   if (table_dtype == DT_F32)
-    embed_gather_kernel<float><<<num_tokens, threads, 0, stream>>>((const float*)table, ids, out, width, vocab);
+    embed_gather_kernel<float><<<num_tokens, threads, 0, stream>>>((const float*)table, ids, out, width, vocab, scale);
   else if (table_dtype == DT_BF16)
-    embed_gather_kernel<bf16><<<num_tokens, threads, 0, stream>>>((const bf16*)table, ids, out, width, vocab);
+    embed_gather_kernel<bf16><<<num_tokens, threads, 0, stream>>>((const bf16*)table, ids, out, width, vocab, scale);
   else
     return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- what a head may still do to its logits ------------------------------------------
+// logits = cap * tanh(scale * logits / cap) (cap 0: only the scale), in place, fp32.  Qwen3 does
+// neither (reference atomserve/model.py:405-415); the decoder launches this only for a plan that
+// names a scale or a cap.
+__global__ void logits_finish_kernel(float* __restrict__ logits, size_t count, float scale, float cap) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+    const float v = logits[i] * scale;
+    logits[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+  }
+}
+
+extern "C" int as_logits_finish(float* logits, long long count, float scale, float cap, hipStream_t stream) {
+  if (count <= 0) return AS_OK;
+  if (cap < 0.f) return AS_BAD_SHAPE;
+  const long long blocks = (count + 255) / 256;
+  logits_finish_kernel<<<(int)(blocks < 2048 ? blocks : 2048), 256, 0, stream>>>(logits, (size_t)count, scale, cap);
   return launch_status();
 }
 
@@ -207,7 +228,7 @@ __global__ void qk_norm_rope_store_kernel(const O* __restrict__ qkv, const W* __
     const size_t head = (size_t)(slot / block_size) * KV + kvh;
     if (!is_k) {  // values: transposed within the page
       O* vt = v_pages + head * block_size * D + slot % block_size;
-      for (int i = lane; i < D; i += WAVE) vt[(size_t)i * block_size] = src[i];
+      for (int i = lane; i < D; i += WAVE) vt[(size_t)i * block_size] = finite_or_zero(src[i]);
       return;
     }
     dst = k_pages + (head * block_size + slot % block_size) * D;
@@ -226,13 +247,15 @@ __global__ void qk_norm_rope_store_kernel(const O* __restrict__ qkv, const W* __
     if (w) { a *= to_f32(w[i]); b *= to_f32(w[i + half]); }
     float c = 1.f, s = 0.f;
     if (cs) { const float2 v = cs[(size_t)t * half + i]; c = v.x; s = v.y; }
-    dst[i] = from_f32<O>(a * c - b * s);
-    dst[i + half] = from_f32<O>(b * c + a * s);
+    const O ra = from_f32<O>(a * c - b * s), rb = from_f32<O>(b * c + a * s);
+    dst[i] = is_k ? finite_or_zero(ra) : ra;
+    dst[i + half] = is_k ? finite_or_zero(rb) : rb;
   }
   for (int i = R + lane; i < D; i += WAVE) {
     float a = to_f32(src[i]) * inv;
     if (w) a *= to_f32(w[i]);
-    dst[i] = from_f32<O>(a);
+    const O ra = from_f32<O>(a);
+    dst[i] = is_k ? finite_or_zero(ra) : ra;
   }
 }
 
@@ -285,8 +308,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_bf16x8_kernel(
       bf16* vt = v_pages + head * block_size * D + slot % block_size;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        vt[(size_t)(8 * l + j) * block_size] = a8[j];
-        vt[(size_t)(half + 8 * l + j) * block_size] = b8[j];
+        vt[(size_t)(8 * l + j) * block_size] = finite_or_zero((bf16)a8[j]);
+        vt[(size_t)(half + 8 * l + j) * block_size] = finite_or_zero((bf16)b8[j]);
       }
       return;
     }
@@ -318,6 +341,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_bf16x8_kernel(
     if (cs) { const float2 v = cs[t * half + 8 * l + j]; c = v.x; sn = v.y; }
     oa[j] = (bf16)(a * c - b * sn);
     ob[j] = (bf16)(b * c + a * sn);
+    if (is_k) { oa[j] = finite_or_zero((bf16)oa[j]); ob[j] = finite_or_zero((bf16)ob[j]); }
   }
   *reinterpret_cast<bf16x8*>(dst + 8 * l) = oa;
   *reinterpret_cast<bf16x8*>(dst + half + 8 * l) = ob;

@@ -13,9 +13,6 @@ import torch
 
 from atomserve_amd.cache.manager import RELEASED
 
-TILE_Q = 64  # query tokens per work item of the prefill attention kernel
-SHORT_ROW = 8  # rows up to this many tokens are attended as single queries (reference runner.py:31-34)
-
 
 @dataclass
 class Row:
@@ -32,6 +29,13 @@ class Row:
     want: list = field(default_factory=list)
     state_slot: int = -1
     store: bool = True
+
+
+def _leading_released(table: list) -> int:
+    n = 0
+    while n < len(table) and table[n] == RELEASED:
+        n += 1
+    return n
 
 
 def slot_of(block_table: list, position: int, block_size: int) -> int:
@@ -64,19 +68,22 @@ class StepBatch:
     token_ids, positions, tok_row [T] int32   (tok_row: which row a token belongs to)
     logits_rows [B'] int32                    flat indices of the wanted positions
     group_slots[g] [T], group_tables[g] [R, W_g] int32, per paged group
-    all_tokens [T]; short_tokens [Ns]: tokens of rows with <= SHORT_ROW tokens;
-    long_tiles [Nt, 4]: (first flat token, count, row, first position) per TILE_Q queries of longer rows
+    all_tokens [T]; with row_split = (short, tile), as the model's mixers ask (`Mixer.row_split`):
+    short_tokens [Ns]: tokens of rows with <= short tokens;
+    long_tiles [Nt, 4]: (first flat token, count, row, first position) per `tile` queries of longer rows
     row_first, row_len, row_start, row_slots [R] int32 (for mixers with per-request state)
     """
 
     def __init__(self, rows, block_size: int, num_paged_groups: int, vocab_size: int, device, pools=None,
-                 staging=None, table_width: int = 0, max_context: int = 0, into=None):  # fmt: skip
+                 staging=None, table_width: int = 0, max_context: int = 0, into=None, row_split=None):  # fmt: skip
         """table_width, max_context: lower bounds that make the layout of a step independent of
         its rows (a step whose kernels were captured in a graph is replayed with new contents).
         into: an earlier batch of identical layout whose device buffer receives this one's arrays."""
         if not rows:
             raise ValueError("a step needs at least one row")
         bs = block_size
+        short_row, tile_q = row_split if row_split is not None else (0, 0)
+        self.row_split = row_split
         tok, pos, trow, want = [], [], [], []
         slots = [[] for _ in range(num_paged_groups)]
         short, tile_list = [], []
@@ -118,12 +125,14 @@ class StepBatch:
             pos.extend(range(row.start, end))
             trow.extend([r] * n)
             want.extend(flat + w for w in row.want)
-            if n <= SHORT_ROW:
+            if row_split is None:
+                pass  # no mixer of this model wants its rows sorted
+            elif n <= short_row:
                 short.extend(range(flat, flat + n))
                 self.max_short_context = max(self.max_short_context, end)
             else:
-                for q0 in range(0, n, TILE_Q):
-                    tile_list.append((flat + q0, min(TILE_Q, n - q0), r, row.start + q0))
+                for q0 in range(0, n, tile_q):
+                    tile_list.append((flat + q0, min(tile_q, n - q0), r, row.start + q0))
             self.max_context = max(self.max_context, end)
             row_first.append(flat)
             row_len.append(n)
@@ -180,6 +189,8 @@ class StepBatch:
             self._at[name] = offset
             offset += a.size
         self._packed = np.concatenate(arrays) if total else np.zeros(0, dtype=np.int32)  # what `advance` edits
+        # per group and row: the leading table entries that a window had given back when this was packed
+        self._given_back = [[_leading_released(row.tables[g]) for row in rows] for g in range(num_paged_groups)]
         self._staging, self._widths, self._vocab = staging, widths, vocab_size
 
         self.num_tokens, self.num_rows = T, R
@@ -225,6 +236,13 @@ class StepBatch:
                 page = row.start // bs
                 p[at[f"slots{g}"] + r] = table[page] * bs + row.start % bs if row.store else -1
                 p[at[f"tables{g}"] + r * self._widths[g] + page] = table[page]
+                # pages that a window has given back since: their ids leave the device's table too
+                # (the kernels skip them, but a tile at the window's edge may still touch one)
+                gone = self._given_back[g][r]
+                while gone < len(table) and gone < self._widths[g] and table[gone] == RELEASED:
+                    p[at[f"tables{g}"] + r * self._widths[g] + gone] = 0
+                    gone += 1
+                self._given_back[g][r] = gone
         total = p.size
         if self._staging is not None:
             host = self._staging.take(total)

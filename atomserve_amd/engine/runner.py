@@ -79,9 +79,16 @@ class DecodeGraphs:
     kernel is this package's; above, the matrix products are the library's, which replay
     correctly (checked against eager steps in the tests, several replays with eager work between).
 
-    All captured steps draw their intermediate tensors from one memory pool (they never run at the
-    same time), so a step holds only its own logits beyond it, 39 MB for 64 rows (155 MB for 256) of a 152K
-    vocabulary; at most `MAX_GRAPHS` are kept, the one replayed longest ago goes first."""
+    A step is captured on rows that pad only (they store nothing and use the state slot that belongs
+    to nobody), so capturing, and the runs that warm it up, touch no request's cache or state; the
+    real rows are packed into the captured buffer afterwards.  A model whose mixers keep a state of
+    their own replays like any other if all its parts say they are capturable.
+
+    All captured steps draw their intermediate tensors from one memory pool and write their logits
+    into one buffer [largest bucket, vocab] (they never run at the same time; a step's logits are
+    read, by the sampling kernels or a copy, before the next step of the same stream overwrites
+    them); at most `MAX_GRAPHS` are kept, the one replayed longest ago goes first.  `bytes_held`
+    is the memory the captures took from the device."""
 
     ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
     CONTEXT_STEP = 1024
@@ -92,14 +99,22 @@ class DecodeGraphs:
         self.graphs = OrderedDict()  # (rows, context) -> (graph, its batch, its logits), least recently used first
         self.pool = None
         self.filler_tables = [[0] for _ in runner.manager.paged_groups]  # one object: a filler row is recognised
+        self.logits = None  # [most_rows, vocab] fp32, shared by all captured steps
+        self.most_rows = _bucket(min(self.ROW_BUCKETS[-1], runner.manager.max_num_seqs), self.ROW_BUCKETS)
+        self.bytes_held = 0
+
+    def filler(self) -> Row:
+        """A row that pads a step: one token at position 0 that stores nothing; if the model keeps
+        per-request state, it works on the slot that belongs to nobody."""
+        slot = self.runner.pools.scrap_slot if self.runner.manager.state_groups else -1
+        return Row([0], 0, self.filler_tables, [0], slot, store=False)
 
     def eligible(self, rows) -> bool:
         r = self.runner
         return (
             r.device.type == "cuda"
             and r.model.capturable
-            and not r.manager.state_groups
-            and 0 < len(rows) <= self.ROW_BUCKETS[-1]
+            and 0 < len(rows) <= self.most_rows
             and all(len(row.tokens) == 1 for row in rows)
         )
 
@@ -114,52 +129,23 @@ class DecodeGraphs:
         width = -(-context // bs)
         # every row of the captured step yields logits; rows that want none are dropped after the replay
         padded = [row if row.want else Row(row.tokens, row.start, row.tables, [0], row.state_slot) for row in rows]
-        padded += [Row([0], 0, self.filler_tables, [0], -1, store=False) for _ in range(n - len(rows))]
+        padded += [self.filler() for _ in range(n - len(rows))]
         key = (n, context)
         entry = self.graphs.get(key)
-        if entry is not None:
-            self.graphs.move_to_end(key)
         if entry is None:
             while len(self.graphs) >= self.MAX_GRAPHS:
                 self.graphs.popitem(last=False)
-            batch = r.prepare(padded, table_width=width, max_context=context)
-            if tokens_from is not None:
-                batch.token_ids[: len(rows)].copy_(tokens_from)
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                r.model.forward(batch)  # loads every library and warms the allocator before capture
-                for _ in range(3):  # and while the library's products are still being tried, again
-                    if not ops.library_trials_pending():
-                        break
-                    r.model.forward(batch)
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            ops.settle_library_choices()  # what the warm-up tried among the library's products is decided now
-            batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
-            graph = torch.cuda.CUDAGraph()
-            if self.pool is None:
-                self.pool = torch.cuda.graph_pool_handle()
-            # No garbage collection while the stream is capturing: a collected object of an
-            # earlier engine (a graph, a tensor) would be destroyed in the middle of the capture,
-            # which the runtime answers by aborting the process.
-            gc.collect()
-            collecting = gc.isenabled()
-            gc.disable()
-            try:
-                with torch.cuda.graph(graph, pool=self.pool):
-                    logits = r.model.forward(batch)
-            finally:
-                if collecting:
-                    gc.enable()
-            entry = self.graphs[key] = (graph, batch, logits)
+            entry = self.graphs[key] = self._capture(n, width, context)
+            fresh = True
         else:
-            if not entry[1].advance(padded):
-                # other requests than last time, or a window moved: pack anew into the captured buffer
-                batch = r.prepare(padded, table_width=width, max_context=context, into=entry[1])
-                entry = self.graphs[key] = (entry[0], batch, entry[2])
-            if tokens_from is not None:
-                entry[1].token_ids[: len(rows)].copy_(tokens_from)
+            self.graphs.move_to_end(key)
+            fresh = False
+        if fresh or not entry[1].advance(padded):
+            # other requests than last time, or a window moved: pack anew into the captured buffer
+            batch = r.prepare(padded, table_width=width, max_context=context, into=entry[1])
+            entry = self.graphs[key] = (entry[0], batch, entry[2])
+        if tokens_from is not None:
+            entry[1].token_ids[: len(rows)].copy_(tokens_from)
         graph, batch, logits = entry
         if r.phases is not None:
             r.phases.mark("pack")
@@ -170,17 +156,55 @@ class DecodeGraphs:
         return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)] if wanted else logits[:0]
 
 
+    def _capture(self, n: int, width: int, context: int):
+        """Captures the decode step of `n` rows and contexts up to `context`, on padding rows."""
+        r = self.runner
+        before = torch.cuda.memory_reserved()
+        if self.logits is None:
+            self.logits = torch.empty((self.most_rows, r.vocab_size), dtype=torch.float32, device=r.device)
+        batch = r.prepare([self.filler() for _ in range(n)], table_width=width, max_context=context)
+        out = self.logits[:n]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            r.model.forward(batch, logits=out)  # loads every library and warms the allocator before capture
+            for _ in range(3):  # and while the library's products are still being tried, again
+                if not ops.library_trials_pending():
+                    break
+                r.model.forward(batch, logits=out)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        ops.settle_library_choices()  # what the warm-up tried among the library's products is decided now
+        batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
+        graph = torch.cuda.CUDAGraph()
+        if self.pool is None:
+            self.pool = torch.cuda.graph_pool_handle()
+        # No garbage collection while the stream is capturing: a collected object of an
+        # earlier engine (a graph, a tensor) would be destroyed in the middle of the capture,
+        # which the runtime answers by aborting the process.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self.pool):
+                r.model.forward(batch, logits=out)
+        finally:
+            if collecting:
+                gc.enable()
+        self.bytes_held += max(0, torch.cuda.memory_reserved() - before)
+        return graph, batch, out
+
     @torch.inference_mode()
     def capture_ahead(self, max_rows: int) -> int:
         """Captures the decode step of every row bucket up to the one that holds `max_rows`, for the
         first context bucket, with rows that store nothing: a server does this once at its start
         instead of pausing when a bucket is first met.  Returns how many graphs were captured."""
-        if not self.eligible([Row([0], 0, self.filler_tables, [0], -1, store=False)]):
+        if not self.eligible([self.filler()]):
             return 0
         before = len(self.graphs)
         for n in self.ROW_BUCKETS:
-            self.run([Row([0], 0, self.filler_tables, [0], -1, store=False) for _ in range(n)])
-            if n >= max_rows:
+            self.run([self.filler() for _ in range(n)])
+            if n >= min(max_rows, self.most_rows):
                 break
         return len(self.graphs) - before
 
@@ -217,6 +241,7 @@ class ModelRunner:
         self.sampler = Sampler(self.device)
         self.staging = Staging(self.device)
         self.vocab_size = model.plan.vocab_size
+        self.row_split = model.row_split()  # how the model's mixers want the rows of a step sorted
         self.decode_graphs = DecodeGraphs(self) if use_graphs else None
         self._token_buffers = []  # pinned, used in turn: the sampled tokens of the steps on their way
         self._token_turn = 0
@@ -224,7 +249,8 @@ class ModelRunner:
 
     def prepare(self, rows, **layout) -> StepBatch:
         return StepBatch(rows, self.manager.block_size, len(self.manager.paged_groups), self.vocab_size,
-                         self.device, pools=self.pools, staging=self.staging, **layout)  # fmt: skip
+                         self.device, pools=self.pools, staging=self.staging, row_split=self.row_split,
+                         **layout)  # fmt: skip
 
     @torch.inference_mode()
     def step(self, rows, tokens_from=None) -> torch.Tensor:
@@ -256,7 +282,11 @@ class ModelRunner:
         """Whether a decode step of these sequences can go to the GPU before the step before it has been
         read: it must be a replayed step, whose token buffer the GPU can fill itself."""
         graphs = self.decode_graphs
-        return graphs is not None and graphs.eligible([Row([0], 0, graphs.filler_tables, [0], -1)] * len(seqs))
+        return graphs is not None and graphs.eligible([graphs.filler()] * len(seqs))
+
+    def graph_bytes(self) -> int:
+        """Device memory that captured decode steps hold (their shared logits and memory pool)."""
+        return 0 if self.decode_graphs is None else self.decode_graphs.bytes_held
 
     @torch.inference_mode()
     def launch(self, out, after: PendingStep = None) -> PendingStep:

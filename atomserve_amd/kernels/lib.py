@@ -7,7 +7,7 @@ library cannot be built or loaded raises.
 """
 
 import ctypes
-from ctypes import c_double, c_float, c_int, c_size_t, c_void_p
+from ctypes import c_double, c_float, c_int, c_longlong, c_size_t, c_void_p
 
 import torch  # noqa: F401  (loads libamdhip64 first)
 
@@ -17,7 +17,8 @@ P, I, F = c_void_p, c_int, c_float
 
 # name -> (library, argument types); every entry point returns an int status.
 SIGNATURES = {
-    "as_embed_gather": ("elementwise", [P, I, P, P, I, I, I, P]),
+    "as_embed_gather": ("elementwise", [P, I, P, P, I, I, I, F, P]),
+    "as_logits_finish": ("elementwise", [P, c_longlong, F, F, P]),
     "as_rmsnorm": ("elementwise", [P, P, P, P, I, F, P, I, I, I, I, P]),
     "as_rope_table": ("elementwise", [P, P, P, I, I, P]),
     "as_qk_norm_rope_store": ("elementwise", [P, I, P, P, I, P, P, P, P, P, I, I, I, I, I, F, I, I, P]),

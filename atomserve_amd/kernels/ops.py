@@ -45,13 +45,22 @@ def _ptr(t) -> int:
     return 0 if t is None else t.data_ptr()
 
 
-def embed_gather(table, ids, out) -> None:
-    """out[t] = table[ids[t]] as fp32.  table [V, h] fp32|bf16, ids [T] int32, out [T, h] fp32."""
+def embed_gather(table, ids, out, scale: float = 1.0) -> None:
+    """out[t] = scale * table[ids[t]] as fp32.  table [V, h] fp32|bf16, ids [T] int32, out [T, h] fp32."""
     _check(table, "table", (F32, BF16), (None, None))
     vocab, width = table.shape
     _check(ids, "ids", I32, (None,))
     _check(out, "out", F32, (ids.shape[0], width))
-    call("as_embed_gather", _ptr(table), _DT[table.dtype], _ptr(ids), _ptr(out), ids.shape[0], width, vocab, _stream())
+    call("as_embed_gather", _ptr(table), _DT[table.dtype], _ptr(ids), _ptr(out), ids.shape[0], width, vocab,
+         float(scale), _stream())  # fmt: skip
+
+
+def logits_finish(logits, scale: float = 1.0, softcap: float = 0.0) -> None:
+    """logits = softcap * tanh(scale * logits / softcap) in place (softcap 0: the scale alone); fp32."""
+    _check(logits, "logits", F32)
+    if softcap < 0:
+        raise KernelError("a soft cap of logits is positive, or 0 for none")
+    call("as_logits_finish", _ptr(logits), logits.numel(), float(scale), float(softcap), _stream())
 
 
 def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True) -> None:
@@ -164,7 +173,8 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
     G = H // KV
-    mfma = q.dtype == BF16 and D % 32 == 0 and G <= 16 and bs % 16 == 0 and not force_generic
+    mfma = (q.dtype == BF16 and D % 32 == 0 and G <= 16 and bs % 16 == 0 and _decode_mfma_fits(D, G)
+            and not force_generic)  # fmt: skip
     part_size, P, part_m, part_l, part_acc = _partitions(N, H, KV, D, max_context, window, mfma, part_size, q.device)
     if mfma:
         call("as_attn_decode_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, _ptr(positions),
@@ -176,7 +186,30 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
          _ptr(part_l), _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 
 
-ATTN_FILL_GROUPS = 384  # (token, kv head) pairs from which on whole contexts beat partitions and their merge (measured)
+DECODE_MFMA_MAX_LDS = 64 << 10  # what a workgroup may ask for without raising the kernel's limit
+
+
+def compute_units() -> int:
+    """Compute units of the current GPU (256 on an MI355X); grids and the fitted costs below scale with it."""
+    global _compute_units
+    if _compute_units is None:
+        _compute_units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    return _compute_units
+
+
+_compute_units = None
+
+
+def _decode_mfma_fits(head_dim: int, group: int) -> bool:
+    """Whether the matrix-core decode kernel's workgroup (queries of a group and four partial outputs
+    in LDS) stays within the LDS a kernel gets unasked; wide heads in large groups do not."""
+    return 4 * (128 + 4 * head_dim * group) + 1024 <= DECODE_MFMA_MAX_LDS
+
+
+def attn_fill_groups() -> int:
+    """(token, kv head) pairs from which on whole contexts beat partitions and their merge: one and a
+    half per compute unit (measured on 256)."""
+    return compute_units() * 3 // 2
 
 
 MFMA_PARTITIONS = (128, 256, 512, 1024, 2048)  # keys per workgroup of the matrix-core decode kernel
@@ -184,12 +217,13 @@ MFMA_PARTITIONS = (128, 256, 512, 1024, 2048)  # keys per workgroup of the matri
 
 def _partition_cost(groups: int, span: int, part: int) -> float:
     """Microseconds, roughly, of the decode attention and its merge when `groups` (token, kv head) pairs
-    cut `span` keys into partitions of `part`: a workgroup costs 4 us and 25 ns a key, 512 of them run
-    at a time, and the merge 0.6 us a partition.  Fitted to the kernel's times at 1 to 32 requests of
-    500 to 33,000 keys (heads of 128, 8 kv heads); what it picks is within 2 per cent of the best
-    partition size on average there, where one size for all was 8 per cent off."""
+    cut `span` keys into partitions of `part`: a workgroup costs 4 us and 25 ns a key, two of them run
+    on a compute unit at a time, and the merge 0.6 us a partition.  Fitted to the kernel's times at 1
+    to 32 requests of 500 to 33,000 keys (heads of 128, 8 kv heads, 256 compute units); what it picks
+    is within 2 per cent of the best partition size on average there, where one size for all was 8 per
+    cent off."""
     parts = math.ceil(span / part)
-    return (4.0 + 0.025 * min(part, span)) * max(1.0, groups * parts / 512) + 0.6 * parts
+    return (4.0 + 0.025 * min(part, span)) * max(1.0, groups * parts / (2 * compute_units())) + 0.6 * parts
 
 
 def _partitions(N, H, KV, D, max_context, window, mfma, part_size, device):
@@ -202,7 +236,7 @@ def _partitions(N, H, KV, D, max_context, window, mfma, part_size, device):
         # the merge stays small; boundaries are multiples of part_size in absolute position.
         if mfma:
             groups = N * KV
-            if groups >= ATTN_FILL_GROUPS:
+            if groups >= attn_fill_groups():
                 part_size = -(-span // 32) * 32  # enough workgroups without partitions: no merge
             else:
                 part_size = min(MFMA_PARTITIONS, key=lambda part: _partition_cost(groups, span, part))
@@ -226,7 +260,8 @@ def attn_decode_fresh_supported(dtype, num_heads: int, num_kv_heads: int, head_d
     """Whether `attn_decode_fresh` takes this case: bfloat16 heads of 64, 128, 192 or 256 with a per-head
     norm, rotated whole, at most 16 query heads to a kv head, pages of a multiple of 16 tokens."""
     return (dtype == BF16 and head_dim % 64 == 0 and head_dim <= 256 and rotary_dim == head_dim and qk_norm
-            and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16 and block_size % 16 == 0)  # fmt: skip
+            and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16 and block_size % 16 == 0
+            and _decode_mfma_fits(head_dim, num_heads // num_kv_heads))  # fmt: skip
 
 
 def attn_decode_fresh(qkv, q_weight, k_weight, cos_sin, slots, eps, store_kv, k_pages, v_pages, positions,
@@ -269,6 +304,7 @@ def attn_decode_fresh(qkv, q_weight, k_weight, cos_sin, slots, eps, store_kv, k_
          _ptr(slots) if store_kv else 0, float(eps), int(bool(store_kv)), _ptr(k_pages), _ptr(v_pages), T,
          _ptr(positions), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
          _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+PREFILL_TILE_QUERIES = 64  # queries of one work item of the prefill kernel
 PREFILL_MAX_HEAD_DIM = 256  # four stages of 32 keys and values of such heads fill 128 KB of LDS
 
 
@@ -308,7 +344,10 @@ SKINNY_TWO_MAX_ROWS, SKINNY_TWO_MAX_K = 32, 4096
 # weights' bytes: at 32 rows of 4096 over 256 workgroups (67 MB) the library's product is faster,
 # with rows of 1024 (17 MB) this one is, by the two kernels it saves beside.
 SKINNY_TWO_MAX_ACT_BYTES = 36 << 20
-WORKGROUPS = 256  # persistent kernels run one workgroup per compute unit
+def _workgroups() -> int:
+    """Persistent kernels run one workgroup per compute unit."""
+    return compute_units()
+
 
 
 def _few_rows(rows: int, k: int, n: int, max_k=None) -> bool:
@@ -318,7 +357,7 @@ def _few_rows(rows: int, k: int, n: int, max_k=None) -> bool:
         return False
     if rows <= SKINNY_MAX_ROWS:
         return max_k is None or k <= max_k
-    strips = min(-(-n // 16), WORKGROUPS)
+    strips = min(-(-n // 16), _workgroups())
     return (rows <= SKINNY_TWO_MAX_ROWS and k <= SKINNY_TWO_MAX_K
             and strips * rows * k * 2 <= SKINNY_TWO_MAX_ACT_BYTES)  # fmt: skip
 
@@ -519,9 +558,9 @@ def gemm_link_supported(rows: int, n_out: int, k: int, dtype) -> bool:
     # two row tiles: the producer reads its activations once per strip of 16 outputs (whole rows
     # for every workgroup of the persistent kernel, and for every strip beyond its K), the consumer
     # keeps rows of n_out in registers in each of its workgroups
-    producer_strips = -(-n_out // 16) if k > SKINNY_TWO_MAX_K else min(-(-n_out // 16), WORKGROUPS)
+    producer_strips = -(-n_out // 16) if k > SKINNY_TWO_MAX_K else min(-(-n_out // 16), _workgroups())
     return (rows <= SKINNY_TWO_MAX_ROWS and producer_strips * rows * k * 2 <= SKINNY_TWO_MAX_ACT_BYTES
-            and _few_rows(rows, n_out, 16 * WORKGROUPS))  # fmt: skip
+            and _few_rows(rows, n_out, 16 * _workgroups()))  # fmt: skip
 
 
 def gemm_link(a, w, x, gain, scaled, ssq) -> None:

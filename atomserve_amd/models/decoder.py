@@ -80,12 +80,20 @@ class DecoderModel:
         return requests
 
     # ---- one pass ---------------------------------------------------------------------
-    def forward(self, step) -> torch.Tensor:
+    def row_split(self):
+        """How the mixers want the rows of a step sorted for their kernels (`Mixer.row_split`): one
+        answer for the whole model, or None if no mixer cares."""
+        wanted = {split for block in self.blocks for split in [block.parts()["mixer"].row_split()] if split is not None}
+        if len(wanted) > 1:
+            raise ValueError(f"the mixers of this model want their rows split in different ways: {sorted(wanted)}")
+        return next(iter(wanted), None)
+
+    def forward(self, step, logits: torch.Tensor = None) -> torch.Tensor:
         """Run this step's tokens through every run of the plan; returns fp32 logits
-        [len(step.logits_rows), vocab] for the wanted rows."""
+        [len(step.logits_rows), vocab] for the wanted rows (written into `logits` if given)."""
         p, dev = self.plan, self.env.device
         x = torch.empty((step.num_tokens, p.hidden_size), dtype=torch.float32, device=dev)
-        ops.embed_gather(self.embed_weight, step.token_ids, x)
+        ops.embed_gather(self.embed_weight, step.token_ids, x, p.embedding_scale)
         delta = None
         for i, r in enumerate(p.run):
             # the norm that the run after this one starts with: this run's last product may add
@@ -94,8 +102,13 @@ class DecoderModel:
             delta = self.blocks[r.layer].forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes),
                                                  next_norm=follows)  # fmt: skip
         n = step.num_logits
-        logits = torch.empty((n, p.vocab_size), dtype=torch.float32, device=dev)
+        if logits is None:
+            logits = torch.empty((n, p.vocab_size), dtype=torch.float32, device=dev)
+        elif logits.shape != (n, p.vocab_size) or logits.dtype != torch.float32:
+            raise ValueError(f"the logits of this step are float32 {(n, p.vocab_size)}, the buffer is {tuple(logits.shape)}")
         if n:
             hf = self.final_norm.forward(x, delta, rows=step.logits_rows, update_residual=False)
             ops.gemm(hf, self.head_weight, logits)
+            if p.logit_scale != 1.0 or p.logit_softcap > 0.0:
+                ops.logits_finish(logits, p.logit_scale, p.logit_softcap)
         return logits

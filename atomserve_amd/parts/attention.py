@@ -14,9 +14,11 @@ import torch
 from atomserve_amd.kernels import ops
 from atomserve_amd.parts.base import Mixer, PagedCacheRequest, PendingNorm, WeightDecl, build, register
 
-# Rows with at most this many new tokens are attended as that many single queries
-# (reference atomserve/runner.py:31-34); longer rows go through the prefill kernel.
+# Rows with at most SHORT_ROW new tokens are attended as that many single queries
+# (reference atomserve/runner.py:31-34); longer rows go through the prefill kernel in work items of
+# TILE_Q consecutive queries.  The step's batch sorts its rows so because this mixer asks for it.
 SHORT_ROW = 8
+TILE_Q = ops.PREFILL_TILE_QUERIES
 
 
 class Attention(Mixer):
@@ -55,6 +57,9 @@ class Attention(Mixer):
     def cache_request(self):
         s = self.spec
         return PagedCacheRequest(s.num_kv_heads, s.head_dim, s.window)
+
+    def row_split(self):
+        return (SHORT_ROW, TILE_Q)
 
     def forward(self, h, step, cache, residual=None, next_norm=None):
         """h [T, hidden] compute dtype (or the norm left pending on the stream) -> [T, hidden], or the
@@ -109,6 +114,8 @@ class Attention(Mixer):
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
                                   cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
             return
+        if step.row_split != self.row_split():
+            raise ValueError(f"this step's rows are sorted as {step.row_split}, the attention kernels need {self.row_split()}")
         if step.num_short_tokens:
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.short_tokens, step.positions, step.tok_row,
                                   cache.block_tables, out, s.scale, s.window, step.max_short_context)  # fmt: skip

@@ -89,7 +89,7 @@ class BuildEnv:
 class PendingNorm:
     """A norm of the fp32 stream `x` whose last step is still due: the part before has added its
     output into `x` and left what the norm's consumer needs to finish the norm inside its first
-    matrix product (`gemm`, `gemm_silu_mul`).  `rows()` runs the norm's own kernel on `x` for a
+    matrix product (`gemm`, `gemm_gated`).  `rows()` runs the norm's own kernel on `x` for a
     consumer that wants the normalised rows themselves."""
 
     def __init__(self, norm: "Norm", x: torch.Tensor):
@@ -103,9 +103,10 @@ class PendingNorm:
         """out = norm(x) @ w^T"""
         raise NotImplementedError
 
-    def gemm_silu_mul(self, w: torch.Tensor, out: torch.Tensor) -> None:
-        """out = silu(norm(x) @ w[:I]^T) * (norm(x) @ w[I:]^T)"""
-        raise NotImplementedError
+    def gemm_gated(self, w: torch.Tensor, out: torch.Tensor, activation: str) -> bool:
+        """out = act(norm(x) @ w[:I]^T) * (norm(x) @ w[I:]^T) in one kernel, if there is one for this
+        activation; else False and nothing done (the caller takes `rows()` and its own kernels)."""
+        return False
 
 
 class Mixer(Part):
@@ -118,6 +119,13 @@ class Mixer(Part):
     adds_to_residual = False
 
     def cache_request(self) -> Optional[Any]:
+        return None
+
+    def row_split(self) -> Optional[tuple]:
+        """(short, tile) if this mixer's kernels want the step's rows sorted: the tokens of rows with
+        at most `short` tokens listed as single queries (`step.short_tokens`), longer rows cut into
+        work items of up to `tile` consecutive tokens (`step.long_tiles`).  None: it reads rows as
+        they come (`step.row_first`, `step.row_len`)."""
         return None
 
     def forward(self, h: torch.Tensor, step: Any, cache: Any) -> torch.Tensor:

@@ -29,10 +29,8 @@ class GatedMLP(FeedForward):
         pending = isinstance(h, PendingNorm)
         T, device = (h.x.shape[0], h.x.device) if pending else (h.shape[0], h.device)
         act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=device)
-        if pending:
-            h.gemm_silu_mul(self.gate_up_weight, act)
-        else:
-            ops.gemm_silu_mul(h, self.gate_up_weight, act)
+        if not (pending and h.gemm_gated(self.gate_up_weight, act, s.activation)):
+            ops.gemm_silu_mul(h.rows() if pending else h, self.gate_up_weight, act)
         if residual is not None and next_norm is not None:
             link = next_norm.absorb(act, self.down_weight, residual)
             if link is not None:

@@ -20,8 +20,11 @@ class PendingRMSNorm(PendingNorm):
     def gemm(self, w, out) -> None:
         ops.gemm_scaled(self.scaled, self.ssq, self.norm.spec.eps, w, out)
 
-    def gemm_silu_mul(self, w, out) -> None:
+    def gemm_gated(self, w, out, activation) -> bool:
+        if activation != "silu":
+            return False
         ops.gemm_scaled(self.scaled, self.ssq, self.norm.spec.eps, w, out, gated=True)
+        return True
 
 
 class RMSNorm(Norm):

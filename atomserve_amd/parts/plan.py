@@ -6,7 +6,7 @@ needs, so no part ever asks which model it is in.  The run list is data too: it 
 name a layer twice, or let a run read the cache that another run writes.
 """
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Any, Optional
 
 
@@ -88,7 +88,9 @@ class ModelPlan:
     final_norm: NormSpec
     tied_head: bool
     max_positions: int
-    extra: dict = field(default_factory=dict)
+    embedding_scale: float = 1.0  # multiplies the embedding rows as they enter the stream
+    logit_scale: float = 1.0  # multiplies the head's output
+    logit_softcap: float = 0.0  # > 0: logits = cap * tanh(logits / cap), after the scale
 
     def cache_id(self, run_index: int) -> int:
         r = self.run[run_index]

@@ -1,8 +1,9 @@
 """Weights from safetensors, by tensor name (reference atomserve/loader.py:63-148).
 
-The architecture says which checkpoint tensors make up each tensor of the plan (q, k,
-v stacked into one projection, gate and up into one); the parts say what shape and
-role each plan tensor has.  Everything that is wrong with a checkpoint is collected
+The architecture says how each tensor of the plan is made of checkpoint tensors: a name,
+names stacked along the rows (q, k, v into one projection, gate and up into one), rows cut
+out of a fused tensor, a transposed matrix, or matrices stacked along a new axis (`Take`,
+`Stack`); the parts say what shape and role each plan tensor has.  Everything that is wrong with a checkpoint is collected
 and reported in one error: missing tensors, unexpected ones, wrong shapes.
 
 Storage: matrices in the compute dtype (bfloat16 when serving); vectors such as norm
@@ -12,12 +13,69 @@ gains keep 32-bit storage when the checkpoint stores them so; integer tables int
 import glob
 import os
 from contextlib import ExitStack
+from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
 _SAFETENSORS_DTYPES = {"F64": torch.float64, "F32": torch.float32, "F16": torch.float16, "BF16": torch.bfloat16,
                        "I64": torch.int64, "I32": torch.int32, "I16": torch.int16, "I8": torch.int8,
                        "U8": torch.uint8, "BOOL": torch.bool}  # fmt: skip
+
+
+@dataclass(frozen=True)
+class Take:
+    """One checkpoint tensor, or a piece of it, as a part of a plan tensor.
+
+    transpose: a matrix stored [in, out] is turned to this package's [out, in] first.
+    rows: (start, stop) keeps these rows only (after the transposition), for a checkpoint that
+    stores several plan tensors fused in one."""
+
+    name: str
+    transpose: bool = False
+    rows: Optional[tuple] = None
+
+    def shape_from(self, stored: tuple) -> tuple:
+        shape = tuple(stored)
+        if self.transpose:
+            if len(shape) != 2:
+                raise ValueError(f"{self.name}: only a matrix can be transposed, this has shape {shape}")
+            shape = shape[::-1]
+        if self.rows is not None:
+            start, stop = self.rows
+            if not 0 <= start < stop <= shape[0]:
+                raise ValueError(f"{self.name}: rows {start}:{stop} lie outside its {shape[0]} rows")
+            shape = (stop - start, *shape[1:])
+        return shape
+
+    def apply(self, tensor):
+        if self.transpose:
+            tensor = tensor.t()
+        if self.rows is not None:
+            tensor = tensor[self.rows[0] : self.rows[1]]
+        return tensor
+
+
+@dataclass(frozen=True)
+class Stack:
+    """Several pieces as one plan tensor: laid one after the other along the rows (q, k and v
+    into one projection), or with `new_axis` as the slices of a new first axis (one matrix per
+    expert into [experts, out, in])."""
+
+    parts: tuple
+    new_axis: bool = False
+
+
+def as_stack(entry) -> Stack:
+    """A checkpoint map's entry in its general form.  An entry may be a checkpoint name, a `Take`,
+    a list of either (stacked along the rows), or a `Stack`."""
+    if isinstance(entry, Stack):
+        parts, new_axis = entry.parts, entry.new_axis
+    elif isinstance(entry, (str, Take)):
+        parts, new_axis = (entry,), False
+    else:
+        parts, new_axis = tuple(entry), False
+    return Stack(tuple(Take(p) if isinstance(p, str) else p for p in parts), new_axis)
 
 
 class WeightsError(ValueError):
@@ -101,19 +159,31 @@ def bind_checkpoint(model, arch, config, source, where: str = "") -> dict:
         raise KeyError(f"architecture {arch.name} maps no checkpoint tensors to {undeclared}")
     present = set(source.names())
     used, missing, wrong = set(), [], []
+    recipes = {target: as_stack(mapping[target]) for target in decls}
     for target, decl in decls.items():
-        sources = mapping[target]
-        used.update(sources)
-        absent = [n for n in sources if n not in present]
+        takes = recipes[target].parts
+        names = [t.name for t in takes]
+        used.update(names)
+        absent = [n for n in names if n not in present]
         missing.extend(absent)
-        for n in sources:
+        bad = False
+        for n in names:
             if n in present and n in expected_shapes and source.shape(n) != tuple(expected_shapes[n][0]):
-                wrong.append((n, source.shape(n), expected_shapes[n][0]))
-        if not absent and not any(w[0] in sources for w in wrong):
-            shapes = [source.shape(n) for n in sources]
-            stacked = (sum(s[0] for s in shapes), *shapes[0][1:])
-            if any(s[1:] != shapes[0][1:] for s in shapes) or stacked != tuple(decl.shape):
-                wrong.append(("+".join(sources), stacked, decl.shape))
+                if not any(w[0] == n for w in wrong):
+                    wrong.append((n, source.shape(n), expected_shapes[n][0]))
+                bad = True
+        if absent or bad:
+            continue
+        shapes = [t.shape_from(source.shape(t.name)) for t in takes]
+        label = "+".join(dict.fromkeys(names))
+        if recipes[target].new_axis:
+            made = (len(shapes), *shapes[0])
+            alike = all(sh == shapes[0] for sh in shapes)
+        else:
+            made = (sum(sh[0] for sh in shapes), *shapes[0][1:])
+            alike = all(sh[1:] == shapes[0][1:] for sh in shapes)
+        if not alike or made != tuple(decl.shape):
+            wrong.append((label, made, decl.shape))
     unexpected = sorted(present - used - set(arch.ignored(config)))
     if missing or unexpected or wrong:
         raise WeightsError(sorted(set(missing)), unexpected, wrong, where)
@@ -121,11 +191,15 @@ def bind_checkpoint(model, arch, config, source, where: str = "") -> dict:
     env = model.env
     tensors = {}
     for target, decl in decls.items():
-        sources = mapping[target]
-        stored = source.dtype(sources[0])
+        recipe = recipes[target]
+        stored = source.dtype(recipe.parts[0].name)
         dtype = _storage_dtype(decl.role, stored, env.dtype)
-        parts = [source.get(n).to(device=env.device, dtype=dtype) for n in sources]
-        tensors[target] = (parts[0] if len(parts) == 1 else torch.cat(parts, dim=0)).contiguous()
+        pieces = [t.apply(source.get(t.name)).to(device=env.device, dtype=dtype) for t in recipe.parts]
+        if recipe.new_axis:
+            made = torch.stack(pieces, dim=0)
+        else:
+            made = pieces[0] if len(pieces) == 1 else torch.cat(pieces, dim=0)
+        tensors[target] = made.contiguous()
     model.bind(tensors)
     return tensors
 

@@ -11,7 +11,7 @@ BS = 4
 
 
 def pack(rows, **layout):
-    return StepBatch(rows, BS, 2, 100, "cpu", **layout)
+    return StepBatch(rows, BS, 2, 100, "cpu", **{"row_split": (8, 64), **layout})
 
 
 def decode_rows(tables, starts, tokens, filler):
@@ -74,3 +74,32 @@ def test_a_repeated_decode_step_is_updated_in_place():
     tables[0][0][2] = 6
     assert batch.advance(decode_rows(tables, [8, 5], [1, 2], filler))
     assert not batch.advance(decode_rows(tables, [12, 6], [1, 2], filler))  # beyond the packed table width
+
+
+def test_rows_are_sorted_only_for_mixers_that_ask():
+    """Short rows and tiles are what the attention kernels of this package want; a model whose
+    mixers ask for nothing gets its rows as they come, another split gives other lists."""
+    rows = [Row([1, 2, 3], 0, [[2], [1]], [2]), Row(list(range(10)), 0, [[3, 0, 6], [4, 5, 7]], [9])]
+    plain = StepBatch(rows, BS, 2, 100, "cpu")
+    assert plain.num_short_tokens == 0 and plain.num_long_tiles == 0
+    assert plain.row_first.tolist() == [0, 3] and plain.row_len.tolist() == [3, 10]
+    split = StepBatch(rows, BS, 2, 100, "cpu", row_split=(2, 4))
+    assert split.num_short_tokens == 0
+    assert sorted(split.long_tiles.tolist()) == [[0, 3, 0, 0], [3, 4, 1, 0], [7, 4, 1, 4], [11, 2, 1, 8]]
+
+
+def test_pages_given_back_by_a_window_leave_the_captured_table():
+    """A request of a windowed group decodes on; the pages its window passes are given back between
+    steps.  The step updated in place holds 0 where packing anew holds 0, not the page's old id
+    (which by then may belong to somebody else)."""
+    filler = [[0]]
+    table = [[5, 2, 7]]
+    first = StepBatch([Row([1], 9, table, [0], -1), Row([0], 0, filler, [0], -1, store=False)], BS, 1, 100, "cpu",
+                      table_width=4, max_context=16)  # fmt: skip
+    table[0][0] = RELEASED
+    table[0][1] = RELEASED
+    rows = [Row([2], 10, table, [0], -1), Row([0], 0, filler, [0], -1, store=False)]
+    assert first.advance(rows)
+    fresh = StepBatch(rows, BS, 1, 100, "cpu", table_width=4, max_context=16)
+    assert torch.equal(first.device_buffer, fresh.device_buffer)
+    assert first.group_tables[0].tolist() == [[0, 0, 7, 0], [0, 0, 0, 0]]

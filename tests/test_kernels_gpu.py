@@ -168,6 +168,69 @@ def test_qk_norm_rope_store_many_tokens_bf16(ops, D, bs, gain, rope):
     assert close_bf16(k_run, ref_k) and torch.equal(v_run.float(), ref_v)
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_what_is_not_finite_never_reaches_the_cache(ops, dtype):
+    """A model that overflows hands the store kernels infinities and NaNs.  Pages are used again by
+    other requests, and kernels multiply masked places by zero, so the pools hold finite values
+    only: what is not finite is stored as zero; finite values and the queries are untouched."""
+    H, KV, D, bs = 4, 2, 64, 16
+    torch.manual_seed(17)
+    qkv = torch.randn(40, H + 2 * KV, D, device=DEV).to(dtype)
+    bad = qkv.clone()
+    bad[3, H, 5] = float("inf")  # a key
+    bad[7, H + KV + 1, 9] = float("nan")  # a value
+    bad[20, H + KV, 0] = float("-inf")  # another value
+    bad[11, H + 1, 63] = 3.0e38 if dtype == BF16 else float("inf")  # finite, and stays so after the norm
+    qw, kw = torch.ones(D, device=DEV, dtype=dtype), torch.ones(D, device=DEV, dtype=dtype)
+    inv = (1.0 / (1e4 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))).to(DEV)
+    cs = torch.empty(40, D // 2, 2, device=DEV)
+    ops.rope_table(i32(list(range(40))), inv, cs)
+    slots = i32(list(range(8, 48)))
+    for weights in ((qw, kw), (None, None)):
+        k_pages = torch.zeros(4, KV, bs, D, dtype=dtype, device=DEV)
+        v_pages = torch.zeros(4, KV, D, bs, dtype=dtype, device=DEV)
+        q = torch.empty(40, H, D, dtype=dtype, device=DEV)
+        ops.qk_norm_rope_store(bad, *weights, cs, slots, q, k_pages, v_pages, H, KV, 1e-6)
+        assert torch.isfinite(k_pages).all() and torch.isfinite(v_pages).all()
+        good_k, good_v, good_q = torch.zeros_like(k_pages), torch.zeros_like(v_pages), torch.empty_like(q)
+        ops.qk_norm_rope_store(qkv, *weights, cs, slots, good_q, good_k, good_v, H, KV, 1e-6)
+        assert torch.equal(q, good_q)
+        clean = torch.ones(40, dtype=torch.bool, device=DEV)
+        clean[[3, 7, 20, 11]] = False
+        rows_k = k_pages.permute(0, 2, 1, 3).reshape(-1, KV, D)[8:48]
+        rows_v = v_pages.permute(0, 3, 1, 2).reshape(-1, KV, D)[8:48]
+        assert torch.equal(rows_k[clean], good_k.permute(0, 2, 1, 3).reshape(-1, KV, D)[8:48][clean])
+        assert torch.equal(rows_v[clean], good_v.permute(0, 3, 1, 2).reshape(-1, KV, D)[8:48][clean])
+        assert rows_v[7, 1, 9] == 0 and rows_v[20, 0, 0] == 0
+
+
+def test_a_decode_step_keeps_the_cache_finite_too(ops):
+    H, KV, D, bs = 8, 2, 128, 16
+    lens = [5, 40, 300]
+    _, k_pages, v_pages, tables, positions = paged_case(BF16, H, KV, D, bs, lens, seed=3)
+    qkv = torch.randn(3, H + 2 * KV, D, device=DEV).to(BF16)
+    qkv[1, H + KV, 7] = float("nan")  # a value of the new token
+    qkv[2, H + 1, 3] = float("inf")  # a coordinate of its key: the norm makes the whole key NaN
+    g = torch.ones(D, device=DEV, dtype=BF16)
+    inv = (1.0 / (1e4 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))).to(DEV)
+    cs = torch.empty(3, D // 2, 2, device=DEV)
+    ops.rope_table(positions, inv, cs)
+    slots = i32([tables[i, (n - 1) // bs].item() * bs + (n - 1) % bs for i, n in enumerate(lens)])
+    out = torch.zeros(3, H, D, dtype=BF16, device=DEV)
+    ops.attn_decode_fresh(qkv, g, g, cs, slots, 1e-6, True, k_pages, v_pages, positions, tables, out, H, D**-0.5, 0, max(lens))
+    torch.cuda.synchronize()
+    assert torch.isfinite(k_pages).all() and torch.isfinite(v_pages).all() and torch.isfinite(out[0]).all()
+
+
+def test_wide_heads_in_large_groups_go_to_the_general_kernel(ops):
+    """16 heads of 256 to one kv head would need more LDS than a workgroup of the matrix-core decode
+    kernel gets: such shapes are routed to the general kernel (test_attention_single_query runs them)
+    and the one-kernel decode step is not offered for them."""
+    assert not ops.attn_decode_fresh_supported(BF16, 16, 1, 256, 16, 256, True)
+    assert ops.attn_decode_fresh_supported(BF16, 16, 2, 256, 16, 256, True)
+    assert ops.attn_decode_fresh_supported(BF16, 16, 1, 128, 16, 128, True)
+
+
 def test_qk_norm_rope_store_variants(ops):
     """No norm, no rotation, a rotation of part of the head, and q alone (a run that reads
     another run's cache stores nothing)."""
@@ -458,7 +521,8 @@ def paged_case(dtype, H, KV, D, bs, lens, seed=0, k_scale=4.0):
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("H,KV,D,bs", [(16, 8, 128, 16), (32, 8, 128, 16), (8, 8, 128, 16), (6, 2, 32, 8),
-                                       (4, 2, 16, 16), (5, 1, 48, 4), (16, 1, 64, 32), (64, 8, 128, 16)])  # fmt: skip
+                                       (4, 2, 16, 16), (5, 1, 48, 4), (16, 1, 64, 32), (64, 8, 128, 16),
+                                       (16, 1, 256, 16), (32, 2, 256, 16)])  # fmt: skip
 def test_attention_single_query(ops, dtype, H, KV, D, bs):
     """Contexts of one key, part of a page, exactly one partition and several partitions, on
     scattered pages (lengths from reference tests/test_kernels.py:98-125)."""
@@ -602,7 +666,7 @@ def test_attention_of_a_batch_that_fills_the_gpu(ops):
     merge), each workgroup walks its whole context, of very different lengths."""
     H, KV, D, bs = 16, 8, 64, 16
     lens = [1 + (37 * i * i) % 1400 for i in range(64)]
-    assert 64 * KV >= ops.ATTN_FILL_GROUPS
+    assert 64 * KV >= ops.attn_fill_groups()
     q, k_pages, v_pages, tables, positions = paged_case(BF16, H, KV, D, bs, lens, seed=5, k_scale=1.0)
     out = torch.zeros(64, H, D, dtype=BF16, device=DEV)
     ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables, out, D**-0.5, 0, max(lens))

@@ -636,8 +636,102 @@ def test_attention_part_alone(dtype):
     outs, at = [], 0
     for n in (20, 1, 1, 8):
         manager.reserve(rc, at, n)
-        batch = StepBatch([Row([0] * n, at, rc.tables, [])], 16, 1, 10, DEV, pools=pools)
+        batch = StepBatch([Row([0] * n, at, rc.tables, [])], 16, 1, 10, DEV, pools=pools, row_split=mixer.row_split())
         outs.append(mixer.forward(x[at : at + n].to(DEV).to(dtype), batch, batch.cache_view(0, True)).float().cpu())
         at += n
     tol = (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(ref.abs().max()))
     assert (torch.cat(outs) - ref).abs().max() <= tol
+
+
+# ---- a mixer with state whose decode steps are captured, and a plan with scaled ends -----------
+
+
+def make_capturable_decay_mixer():
+    base = make_decay_mixer()
+
+    class DecayMixerOnDevice(base):
+        """The same running sum; a step in which every row brings one token is computed from the
+        step's device arrays alone (slots, first positions), so it can be captured and replayed.
+        Rows that pad a captured step arrive with the slot that belongs to nobody."""
+
+        capturable = True
+
+        def forward(self, h, step, cache):
+            if not step.decode_only:
+                return super().forward(h, step, cache)
+            slots = step.row_slots.long()
+            old = torch.where((step.row_start == 0)[:, None], torch.zeros((), device=h.device), cache.state[slots])
+            s = old * self.spec.decay + h.float()
+            cache.state.index_copy_(0, slots, s)
+            return (s * self.gain.float()).to(h.dtype)
+
+    return DecayMixerOnDevice
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_steps_of_a_mixer_with_state_are_captured_and_replayed(dtype, device=DEV):
+    """A model with a state of its own per request decodes through captured steps like any other,
+    once its parts say they can be captured: the capture and its warm-up runs work on padding rows
+    and the slot that belongs to nobody, so no request's state moves before its step is replayed."""
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.parts.base import register
+
+    arch = register_toy_architecture()
+    register("mixer", "toy_decay", make_capturable_decay_mixer(), replace=True)
+    raw = {**TINY_B, "architectures": ["ToyDecayForCausalLM"], "num_hidden_layers": 4}
+    w = plain_random_weights(raw, seed=5, std=0.2, gain_std=0.2)
+    for i in (1, 3):
+        for k in [k for k in w if k.startswith(f"model.layers.{i}.self_attn.")]:
+            del w[k]
+        w[f"model.layers.{i}.decay.gain"] = (1 + 0.2 * torch.randn(raw["hidden_size"])).bfloat16().float()
+    engine = build_engine(arch, raw, w, dtype, device)
+    assert engine.runner.model.capturable and engine.scheduler.manager.state_groups
+    prompts = [torch.randint(0, 1000, (n,), generator=torch.Generator().manual_seed(n)).tolist() for n in (7, 12, 1)]
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True))
+    graphs = engine.runner.decode_graphs.graphs
+    assert graphs and engine.counters["steps"] >= 9
+    assert engine.scheduler.manager.num_free_slots == 4
+    for prompt, out in zip(prompts, outs):
+        seq = list(prompt)
+        for t in out:
+            ref = plain_toy_logits(raw, w, seq)[-1]
+            if dtype == torch.float32:
+                assert t == int(ref.argmax())
+            else:
+                assert ref[t] >= ref.max() - 6e-2 * max(1.0, float(ref.abs().max()))
+            seq.append(t)
+    register("mixer", "toy_decay", make_decay_mixer(), replace=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_plan_scales_its_embeddings_and_caps_its_logits(dtype, device=DEV):
+    """Embedding multiplier, logit scale and soft cap are fields of the plan that the decoder reads;
+    Qwen3 leaves them at 1, 1 and none."""
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+
+    qwen = architecture_for(TINY_A)
+    scale_in, scale_out, cap = 3.0, 1.5, 4.0
+
+    def build_plan(c):
+        return dataclasses.replace(qwen.build_plan(c), embedding_scale=scale_in, logit_scale=scale_out, logit_softcap=cap)
+
+    arch = register_architecture(
+        Architecture("ScaledForCausalLM", qwen.parse_config, build_plan, qwen.checkpoint_map, qwen.checkpoint_shapes), replace=True
+    )
+    raw = {**TINY_A, "architectures": ["ScaledForCausalLM"]}
+    w = plain_random_weights(raw, seed=12, std=0.2, gain_std=0.2)
+    engine = build_engine(arch, raw, w, dtype, device)
+    ids = torch.randint(0, 256, (30,), generator=torch.Generator().manual_seed(7)).tolist()
+    scaled = dict(w)
+    scaled["model.embed_tokens.weight"] = w["model.embed_tokens.weight"] * scale_in  # tied: the head is the unscaled table
+    hidden = plain.hidden_states(raw, scaled, ids)
+    hidden = plain.rms_norm(hidden, w["model.norm.weight"].double(), raw["rms_norm_eps"])
+    uncapped = hidden @ w["model.embed_tokens.weight"].double().T * scale_out
+    ref = (cap * torch.tanh(uncapped / cap)).float()
+    caches = {}
+    got = torch.cat([step_rows(engine, caches, [("a", ids[:20], list(range(20)))])]
+                    + [step_rows(engine, caches, [("a", [ids[i]], [0])]) for i in range(20, 30)])  # fmt: skip
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    # the cap's slope is at most one: an error of the scaled logits passes through no larger
+    assert (got - ref).abs().max() <= tol * max(1.0, float(uncapped.abs().max()))
+    assert 0.7 * cap < ref.abs().max() < cap  # the cap bites

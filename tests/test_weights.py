@@ -112,3 +112,68 @@ def test_sharded_folder_is_read_across_files(tmp_path):
     save_file({k: w[k].bfloat16() for k in names[1::2]}, os.path.join(path, "model-00002-of-00002.safetensors"))
     model, _, _ = load_model(path, torch.float32, "cpu")
     assert torch.equal(model.embed_weight, w["model.embed_tokens.weight"])
+
+
+def test_a_checkpoint_of_another_layout_is_a_matter_of_the_map_alone():
+    """The same model from a checkpoint that fuses q, k and v in one tensor, stores gate and up fused
+    in the other order, keeps the output projection transposed ([in, out]) and, for a part with
+    experts, one matrix per expert: the architecture's map names slices, a transposition and a stack
+    along a new axis; the loader itself does not change."""
+    import dataclasses
+
+    from atomserve_amd.config.registry import Architecture, architecture_for
+    from atomserve_amd.models.decoder import DecoderModel
+    from atomserve_amd.weights import Stack, Take
+    from atomserve_amd.weights.loader import DictSource, bind_checkpoint
+
+    raw = dict(TINY_B, num_hidden_layers=1)
+    qwen = architecture_for(raw)
+    c = qwen.parse_config(raw)
+    w = plain_random_weights(raw, seed=3)
+    p, inter = "model.layers.0.", c.intermediate_size
+    other = {k: v for k, v in w.items() if "_proj" not in k}
+    other[p + "attn.c_attn"] = torch.cat([w[p + f"self_attn.{x}_proj.weight"] for x in "qkv"])
+    other[p + "attn.c_proj"] = w[p + "self_attn.o_proj.weight"].t().contiguous()
+    other[p + "mlp.up_gate"] = torch.cat([w[p + "mlp.up_proj.weight"], w[p + "mlp.gate_proj.weight"]])
+    other[p + "mlp.down_proj.weight"] = w[p + "mlp.down_proj.weight"]
+
+    def checkpoint_map(cfg):
+        names = qwen.checkpoint_map(cfg)
+        names["layers.0.mixer.qkv.weight"] = p + "attn.c_attn"
+        names["layers.0.mixer.o.weight"] = Take(p + "attn.c_proj", transpose=True)
+        names["layers.0.ffn.gate_up.weight"] = [Take(p + "mlp.up_gate", rows=(inter, 2 * inter)),
+                                                Take(p + "mlp.up_gate", rows=(0, inter))]  # fmt: skip
+        return names
+
+    arch = Architecture("Other", qwen.parse_config, qwen.build_plan, checkpoint_map, lambda cfg: {})
+    model = DecoderModel(arch.build_plan(c), torch.float32, "cpu")
+    bind_checkpoint(model, arch, c, DictSource(other))
+    reference = DecoderModel(qwen.build_plan(c), torch.float32, "cpu")
+    bind_checkpoint(reference, qwen, c, DictSource(w))
+    assert model._tensors.keys() == reference._tensors.keys()
+    for name, t in reference._tensors.items():
+        assert torch.equal(model._tensors[name], t), name
+
+    # a transposed tensor of the wrong size and a slice beyond the tensor are named in the one error
+    broken = dict(other)
+    broken[p + "attn.c_proj"] = torch.zeros(5, 7)
+    with pytest.raises(WeightsError, match="attn.c_proj is \\(7, 5\\), expected"):
+        bind_checkpoint(DecoderModel(arch.build_plan(c), torch.float32, "cpu"), arch, c, DictSource(broken))
+
+    # matrices of three experts stacked along a new first axis
+    class Experts:
+        env = model.env
+
+        def weight_decls(self):
+            from atomserve_amd.parts.base import WeightDecl
+
+            return {"experts.weight": WeightDecl((3, 4, 6))}
+
+        def bind(self, tensors):
+            self.tensors = tensors
+
+    mats = {f"expert.{i}.w": torch.randn(4, 6) for i in range(3)}
+    toy = dataclasses.replace(arch, checkpoint_map=lambda cfg: {"experts.weight": Stack(tuple(mats), new_axis=True)})
+    holder = Experts()
+    bind_checkpoint(holder, toy, c, DictSource(mats))
+    assert torch.equal(holder.tensors["experts.weight"], torch.stack(list(mats.values())))
