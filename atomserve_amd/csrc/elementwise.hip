@@ -306,6 +306,41 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_bf16x8_kernel(
     const size_t head = (size_t)(slot / block_size) * KV + kvh;
     if (!is_k) {  // values: transposed within the page
       bf16* vt = v_pages + head * block_size * D + slot % block_size;
+      // A prompt's tokens fill a page slot after slot.  Where eight tokens in a row go to eight
+      // slots in a row that start at a multiple of eight, the first of them stores for all:
+      // a coordinate's eight values are 16 contiguous bytes of the transposed page, where token
+      // by token they would be eight stores of two bytes, 2 * block_size bytes apart.
+      const long lead = (long)t - (slot & 7);
+      bool run = (block_size & 7) == 0 && lead >= 0 && lead + 8 <= (long)(units / heads);
+      if (run) {
+        const int first = slot - (slot & 7);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) run = run && slots[lead + i] == first + i;
+      }
+      if (run) {  // uniform over the lanes of this (token, head)
+        if (slot & 7) return;  // the first token of the eight does it
+        bf16x8 va[8], vb[8];
+        va[0] = a8;
+        vb[0] = b8;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+          const bf16* si = src + (size_t)i * (H + 2 * KV) * D;
+          va[i] = *reinterpret_cast<const bf16x8*>(si + 8 * l);
+          vb[i] = *reinterpret_cast<const bf16x8*>(si + half + 8 * l);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          bf16x8 oa, ob;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            oa[i] = finite_or_zero((bf16)va[i][j]);
+            ob[i] = finite_or_zero((bf16)vb[i][j]);
+          }
+          *reinterpret_cast<bf16x8*>(vt + (size_t)(8 * l + j) * block_size) = oa;
+          *reinterpret_cast<bf16x8*>(vt + (size_t)(half + 8 * l + j) * block_size) = ob;
+        }
+        return;
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         vt[(size_t)(8 * l + j) * block_size] = finite_or_zero((bf16)a8[j]);

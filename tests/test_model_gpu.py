@@ -142,6 +142,30 @@ def test_configurations_drawn_at_random(seed, tmp_path):
             check(worst, scale, dtype)
 
 
+def test_the_error_of_bfloat16_is_what_rounding_alone_does(setup):
+    """The bound of the bfloat16 tests above is a few rounding steps of the largest logit.  This one
+    is calibrated: the plain model with its activations rounded to bfloat16 at the places where an
+    engine that stores them so must round (tests/plain_qwen3.py `storage`) moves away from the exact
+    logits by some root mean square; the engine, whole prompts and decoded tokens alike, is no
+    further from the exact logits than one and a half times that, over all logits of a request."""
+    name, raw, weights, path, cache = setup
+    ids = rc.random_ids(raw["vocab_size"], LENGTHS[name], seed=1)
+    exact = plain.logits(raw, weights, ids, batched=True).float()
+    rounded = plain.logits(raw, weights, ids, batched=True, storage=torch.bfloat16).float()
+    noise = float((rounded - exact).pow(2).mean().sqrt())
+    for steps in (rc.whole("a", ids), rc.prefill_then_decode("a", ids, tail=64), rc.portions("a", ids)):
+        replay = make_replay(path, "bfloat16", rc.live_token_bound(steps), PAGE[name])
+        at, sq, n = 0, 0.0, 0
+        for s in steps:
+            logits = replay.step(s["entries"], s["end"])
+            e = s["entries"][0]
+            for k, w in enumerate(e["want"]):
+                sq += float((logits[k] - exact[at + w]).pow(2).sum())
+                n += exact.shape[1]
+            at += len(e["tokens"])
+        assert n and (sq / n) ** 0.5 <= 1.5 * noise, f"engine {(sq / n) ** 0.5:.3e} against rounding {noise:.3e}"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_and_long_decoding(setup, dtype):
     name, raw, weights, path, cache = setup
@@ -405,6 +429,40 @@ def test_decode_steps_sent_ahead_give_the_same_tokens(setup, dtype):
     assert {reason for _, reason in waited} >= {"stop", "length", "abort"}
 
 
+def test_steps_sent_ahead_while_the_batch_shrinks_across_kernel_choices(setup):
+    """Seventeen and thirty-three requests decode while some stop on a token: a request that has
+    stopped rides one step too many, so the steps sent ahead cross from 17 rows to 16 and from 33 to
+    32 (other row buckets, other matrix-product kernels) one step later than an engine that waits.
+    In 32-bit every token is the same either way."""
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.weights import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, torch.float32, "cuda:0")
+    vocab = raw["vocab_size"]
+    eos = frozenset(range(0, vocab, 23))
+    for count in (17, 33):
+        prompts = [rc.random_ids(vocab, 3 + (7 * i) % 20, seed=900 + i) for i in range(count)]
+        params = [SamplingParams(temperature=0.8 if i % 3 else 0.0, top_k=15, max_tokens=20 + i % 5, seed=i, ignore_eos=i % 4 == 0)
+                  for i in range(count)]  # fmt: skip
+        results = []
+        for run_ahead in (False, True):
+            cfg = EngineConfig(block_size=16, num_blocks=160, max_model_len=64, max_num_seqs=40, max_num_batched_tokens=512)
+            engine = create_engine(model, cfg, eos)
+            engine.run_ahead = run_ahead
+            handles = [engine.submit(p, q) for p, q in zip(prompts, params)]
+            sizes = set()
+            while engine.step():
+                sizes.add(engine.counters["last_batch_seqs"])
+            results.append([(list(h), h.finish_reason) for h in handles])
+            assert engine.stats()["kv_blocks_used"] == 0
+            assert count in sizes and min(sizes) < count - 1  # the batch did shrink across the boundary
+        assert results[0] == results[1]
+        assert {"stop", "length"} <= {reason for _, reason in results[0]}
+
+
 def test_a_step_sent_ahead_may_be_the_first_of_its_graph(tmp_path):
     """Requests that decode from 1,015 and 1,020 tokens pass the context bound of the captured steps
     while steps are sent ahead: the step that is captured anew takes its tokens from the GPU like
@@ -494,7 +552,27 @@ def test_command_line_generates(setup, capsys):
     assert main([path, "--random-weights", "3", "--temperature", "0.7", "--seed", "1", "--max-tokens", "4", "--prompt-ids", "1 2 3",
                  "--kv-mem-gb", "0.01", "--max-num-seqs", "4", "--max-batched-tokens", "16"]) == 0  # fmt: skip
     out = [js.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
-    assert len(out) == 1 and len(out[0]["output_ids"]) <= 4
+    assert len(out) == 1 and 1 <= len(out[0]["output_ids"]) <= 4
+    assert all(0 <= t < raw["vocab_size"] for t in out[0]["output_ids"])
+    # weights from a seed, greedy, 32-bit: the tokens are the plain model's on the same drawn weights
+    from atomserve_amd.config.registry import architecture_for
+    from atomserve_amd.weights.random_init import random_checkpoint
+
+    arch = architecture_for(raw)
+    drawn = random_checkpoint(arch, arch.parse_config(raw), 3, dtype=torch.float32, device="cuda:0")
+    drawn = {k: v.cpu() for k, v in drawn.items()}
+    assert main([path, "--random-weights", "3", "--dtype", "fp32", "--temperature", "0", "--max-tokens", "4", "--ignore-eos",
+                 "--prompt-ids", "1 2 3", "--kv-mem-gb", "0.01", "--max-num-seqs", "4", "--max-batched-tokens", "16"]) == 0  # fmt: skip
+    out = [js.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert out[0]["output_ids"] == plain.greedy(raw, drawn, [1, 2, 3], 4)
+    # the same seed and settings twice: the same sampled tokens
+    runs = []
+    for _ in range(2):
+        assert main([path, "--random-weights", "3", "--dtype", "fp32", "--temperature", "0.9", "--seed", "5", "--max-tokens", "6",
+                     "--ignore-eos", "--prompt-ids", "4 5", "--kv-mem-gb", "0.01", "--max-num-seqs", "4",
+                     "--max-batched-tokens", "16"]) == 0  # fmt: skip
+        runs.append([js.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")][0]["output_ids"])
+    assert runs[0] == runs[1] and len(runs[0]) == 6
 
 
 def test_engine_thread_under_concurrent_clients(setup):
