@@ -57,20 +57,38 @@ extern "C" int as_logits_finish(float* logits, long long count, float scale, flo
 //   v = x[s] + (delta ? delta[s] : 0)          in fp32; written back to x[s] if update_x
 //   out[r] = v / sqrt(mean(v^2) + eps) * w     rounded once
 // Plain reference: reference atomserve/model.py:125-139 (weight multiplies directly).
+//
+// The pending sum may also arrive as the partial sums of a matrix product whose K was cut into
+// `splits` ranges (SplitDelta: fp32 [splits, rows, n]): they are added in the order of the ranges
+// and rounded to O once, which is what the product alone would have stored.
+struct SplitDelta {
+  const float* sums;  // null: none
+  int splits;
+  size_t stride;  // elements from one range's sums to the next: rows * n
+};
+
+template <typename O>
+__device__ __forceinline__ float split_delta(const SplitDelta& sd, size_t at) {
+  float d = sd.sums[at];
+  for (int k = 1; k < sd.splits; ++k) d += sd.sums[(size_t)k * sd.stride + at];
+  return to_f32(from_f32<O>(d));
+}
+
 template <typename O, typename W>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const O* __restrict__ delta,
                                const int* __restrict__ rows, const W* __restrict__ w, float eps,
-                               O* __restrict__ out, int n, int update_x) {
+                               O* __restrict__ out, int n, int update_x, SplitDelta sd) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t s = rows ? (size_t)rows[r] : (size_t)r;
   float* xr = x + s * n;
   const O* dr = delta ? delta + s * n : nullptr;
+  const bool pending = dr || sd.sums;
   float ss = 0.f;
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     float v = xr[i];
-    if (dr) {
-      v += to_f32(dr[i]);
+    if (pending) {
+      v += dr ? to_f32(dr[i]) : split_delta<O>(sd, s * n + i);
       if (update_x) xr[i] = v;
     }
     ss += v * v;
@@ -80,7 +98,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const O* __restrict__ delt
   O* o = out + (size_t)r * n;
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     float v = xr[i];  // the thread's own earlier store, if any, is what it reads back
-    if (dr && !update_x) v += to_f32(dr[i]);
+    if (pending && !update_x) v += dr ? to_f32(dr[i]) : split_delta<O>(sd, s * n + i);
     o[i] = from_f32<O>(v * inv * to_f32(w[i]));
   }
 }
@@ -110,7 +128,8 @@ template <typename O, typename W>
 __global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ x, const O* __restrict__ delta,
                                                            const int* __restrict__ rows,
                                                            const W* __restrict__ w, float eps,
-                                                           O* __restrict__ out, int n, int update_x) {
+                                                           O* __restrict__ out, int n, int update_x,
+                                                           SplitDelta sd) {
   __shared__ float red[17];
   const int r = blockIdx.x;
   const size_t s = rows ? (size_t)rows[r] : (size_t)r;
@@ -124,8 +143,20 @@ __global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ x
     const int c = threadIdx.x + j * blockDim.x;
     if (c < chunks) {
       v[j] = Vec4<float>::load(xr + 4 * c);
-      if (dr) {
-        const float4 d = Vec4<O>::load(dr + 4 * c);
+      if (dr || sd.sums) {
+        float4 d;
+        if (dr) {
+          d = Vec4<O>::load(dr + 4 * c);
+        } else {
+          const float* p = sd.sums + s * n + 4 * c;
+          d = Vec4<float>::load(p);
+          for (int k = 1; k < sd.splits; ++k) {
+            const float4 e = Vec4<float>::load(p + (size_t)k * sd.stride);
+            d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+          }
+          d = make_float4(to_f32(from_f32<O>(d.x)), to_f32(from_f32<O>(d.y)), to_f32(from_f32<O>(d.z)),
+                          to_f32(from_f32<O>(d.w)));
+        }
         v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
         if (update_x) Vec4<float>::store(xr + 4 * c, v[j]);
       }
@@ -145,8 +176,8 @@ __global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(float* __restrict__ x
   }
 }
 
-extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const void* w, int w_dtype,
-                          float eps, void* out, int out_dtype, int num_out_rows, int n, int update_x,
+static int launch_rmsnorm(float* x, const void* delta, const SplitDelta& sd, const int* rows, const void* w,
+                          int w_dtype, float eps, void* out, int out_dtype, int num_out_rows, int n, int update_x,
                           hipStream_t stream) {
   if (num_out_rows <= 0) return AS_OK;
   if (n <= 0) return AS_BAD_SHAPE;
@@ -163,10 +194,10 @@ extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const vo
   do {                                                                                             \
     if (vec)                                                                                       \
       rmsnorm_vec_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)delta, rows, (const W*)w, eps, \
-                                                                     (O*)out, n, update_x);        \
+                                                                     (O*)out, n, update_x, sd);    \
     else                                                                                           \
       rmsnorm_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)delta, rows, (const W*)w, eps,     \
-                                                                 (O*)out, n, update_x);            \
+                                                                 (O*)out, n, update_x, sd);        \
   } while (0)
   if (out_dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
   else if (out_dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
@@ -174,6 +205,23 @@ extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const vo
   else return AS_BAD_DTYPE;
 #undef LAUNCH
   return launch_status();
+}
+
+extern "C" int as_rmsnorm(float* x, const void* delta, const int* rows, const void* w, int w_dtype,
+                          float eps, void* out, int out_dtype, int num_out_rows, int n, int update_x,
+                          hipStream_t stream) {
+  return launch_rmsnorm(x, delta, SplitDelta{nullptr, 0, 0}, rows, w, w_dtype, eps, out, out_dtype, num_out_rows, n,
+                        update_x, stream);
+}
+
+// The same with the pending sum given as the partial sums [splits, num_rows, n] (fp32) of a product
+// whose K was cut into ranges; num_rows counts the rows of x.
+extern "C" int as_rmsnorm_split(float* x, const float* sums, int splits, int num_rows, const int* rows, const void* w,
+                                int w_dtype, float eps, void* out, int out_dtype, int num_out_rows, int n,
+                                int update_x, hipStream_t stream) {
+  if (!sums || splits <= 0 || num_rows <= 0) return AS_BAD_SHAPE;
+  return launch_rmsnorm(x, nullptr, SplitDelta{sums, splits, (size_t)num_rows * n}, rows, w, w_dtype, eps, out,
+                        out_dtype, num_out_rows, n, update_x, stream);
 }
 
 // ---- rotary table -------------------------------------------------------------------

@@ -87,6 +87,8 @@ extern "C" int as_gemm_f32(const float* a, const float* w, float* out, int M, in
 // Needs K % 8 == 0 (16-byte loads).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+// s_waitcnt that only constrains the vector-memory counter (vmcnt: bits 3:0 and 15:14)
+#define PF_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 
 template <typename OutT> __device__ __forceinline__ void store4(OutT* p, floatx4 v, int valid);
@@ -509,6 +511,240 @@ extern "C" int as_gemm_bf16_scaled(const void* scaled, const float* ssq, int str
                : dispatch_pipe<false, bf16, true, false>(scaled, w, out, M, N, K, stream, link);
 }
 
+// ---- bf16, 17 to 64 rows: tiles of weight rows with the activations staged in LDS ----------
+//
+// With more than 16 rows the activations no longer fit a wave's registers, and reading them from
+// memory again for every strip of 16 weight rows costs as much as reading weights (a 16-byte load
+// per lane costs the same whether it ends in L2 or in HBM).  Here a workgroup of 8 waves owns NS
+// strips (NS = 8, 4 or 2; 8 / NS waves share a strip and split every chunk of K between them) and
+// walks K in chunks of 256: the chunk's activations come into LDS once per workgroup by loads that
+// pass through registers (requested one chunk ahead, in LDS for the chunk in use and the one
+// before), every wave multiplies its strip's weights (straight from memory into registers, two
+// chunks ahead) with them.  So a workgroup reads M rows of
+// activations for 16 NS rows of weights; fewer strips make more workgroups where N is small.
+//
+//   GATED:   the first half of the strips are gate rows, the second half the up rows of the same
+//            outputs; the up sums meet the gate sums in LDS and out = silu(gate) * up, both rounded
+//            to OutT first.
+//   PARTIAL: blockIdx.y names a range of K; the fp32 sums of that range go to
+//            partial[split][m][n] for whoever adds the ranges up (the RMSNorm that follows does).
+//
+// LDS slot (16 bytes) of activation row r, k-block c (8 values) of a chunk: r * 32 + (c ^ (r & 15)):
+// the 16 rows that the lanes of an MFMA operand read at one k-block lie in 16 different bank groups.
+// Needs K % 256 == 0 (and ranges of K that are multiples of 256).
+constexpr int TILE_KC = 256;
+constexpr int tile_waves(int ns) { return ns == 6 ? 6 : 8; }
+constexpr int TILE_RING = 2;
+
+template <int MT, int NS, bool GATED, bool PARTIAL, typename OutT>
+__global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(const bf16* __restrict__ a,
+                                                                        const bf16* __restrict__ w,
+                                                                        OutT* __restrict__ out,
+                                                                        float* __restrict__ partial, int M, int N,
+                                                                        int K, int k_per_split) {
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* global_ptr_t;
+  constexpr int TILE_WAVES = tile_waves(NS), NT = TILE_WAVES * 64;
+  constexpr int KW = TILE_WAVES / NS;  // waves that share a strip
+  constexpr int STEPS = 4 / KW;        // 64-wide steps of a chunk that one wave multiplies
+  constexpr int ROWS = MT * 16, SLOTS = ROWS * 32;  // 16-byte slots of one chunk
+  constexpr int OUT_STRIPS = GATED ? NS / 2 : NS;   // strips of outputs per workgroup
+  constexpr int COPIES = (SLOTS + NT - 1) / NT;  // 16-byte pieces of a chunk that one thread moves
+  static_assert(NS == 8 || NS == 6 || NS == 4 || NS == 2, "8 waves divide into 8, 4 or 2 strips of 16 rows; 6 waves take 6");
+  extern __shared__ __attribute__((aligned(16))) u32x4_t tile_lds[];  // [TILE_RING][SLOTS]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const int strip = wave % NS, kw = wave / NS;
+  const int k0 = PARTIAL ? blockIdx.y * k_per_split : 0;
+  const int k1 = PARTIAL ? min(K, k0 + k_per_split) : K;
+  const int nchunks = (k1 - k0) / TILE_KC;
+  // this wave's 16 weight rows (rows beyond N repeat the last one; their sums are not stored)
+  const bool is_up = GATED && strip >= OUT_STRIPS;
+  const int n0 = blockIdx.x * (16 * OUT_STRIPS) + (strip % OUT_STRIPS) * 16;  // first output column of the strip
+  // Loads go through buffer descriptors: a load beyond the buffer's end returns zeros and moves no
+  // data, so every chunk issues the same loads (those for chunks past the last are sent beyond the
+  // end) and the count of loads in flight at any point of the loop is known exactly.
+  const unsigned w_rows = (unsigned)(GATED ? 2 * N : N);
+  const __amdgpu_buffer_rsrc_t w_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16*>(w), 0, (int)(w_rows * (unsigned)K * 2u), 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16*>(a), 0, (int)((unsigned)M * (unsigned)K * 2u), 0x00020000);
+  constexpr unsigned BEYOND = 0xfffffff0u;
+  const unsigned w_off = (((unsigned)min(n0 + lr, N - 1) + (is_up ? (unsigned)N : 0u)) * (unsigned)K + k0 + lg * 16) * 2u;
+
+  // ---- activations: chunk j travels through registers (requested one chunk ahead, 16-byte loads
+  // spread over the threads) into LDS slot j % 2 just before it is used
+  u32x4_t held[COPIES];
+  unsigned a_off[COPIES];
+#pragma unroll
+  for (int i = 0; i < COPIES; ++i) {
+    const int slot = i * NT + tid, r = slot >> 5, c = (slot & 31) ^ (r & 15);
+    a_off[i] = slot < SLOTS ? ((unsigned)min(r, M - 1) * (unsigned)K + k0 + c * 8) * 2u : BEYOND;
+  }
+  auto request = [&](int j) {
+#pragma unroll
+    for (int i = 0; i < COPIES; ++i)
+      held[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          a_buf, (j < nchunks && a_off[i] != BEYOND) ? a_off[i] + j * (TILE_KC * 2) : BEYOND, 0, 0);
+  };
+  auto deposit = [&](int j) {
+    u32x4_t* dst = tile_lds + (j % TILE_RING) * SLOTS + tid;
+#pragma unroll
+    for (int i = 0; i < COPIES; ++i)
+      if (SLOTS % NT == 0 || i * NT + tid < SLOTS) dst[i * NT] = held[i];
+  };
+  // Three sets of registers hold the weights of this chunk, the next and the one after; their
+  // roles rotate with the chunks (copying one set into another would wait for the newest loads).
+  u32x4_t wa[STEPS][2], wb[STEPS][2], wc[STEPS][2];
+  auto fetch = [&](u32x4_t (&into)[STEPS][2], int j) {
+    const unsigned base = j < nchunks ? w_off + j * (TILE_KC * 2) : BEYOND;
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+      const unsigned at = j < nchunks ? base + (kw + i * KW) * 128 : BEYOND;
+      into[i][0] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, at, 0, 0);
+      into[i][1] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, j < nchunks ? at + 16 : BEYOND, 0, 0);
+    }
+  };
+  floatx4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // One chunk: its activations (in registers by now) go to LDS, whose slot everyone left before the
+  // barrier of the chunk before; the next chunk's activations and the weights of the chunk after
+  // next are requested; a bare barrier (a fence would wait for every load in flight); the products.
+  auto chunk = [&](int j, u32x4_t (&now)[STEPS][2], u32x4_t (&later)[STEPS][2]) {
+    deposit(j);
+    request(j + 1);
+    fetch(later, j + 2);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
+    __builtin_amdgcn_s_barrier();
+    const u32x4_t* acts = tile_lds + (j % TILE_RING) * SLOTS;
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int c = (kw + i * KW) * 8 + lg * 2 + h;
+        const bf16x8 wv = __builtin_bit_cast(bf16x8, now[i][h]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const bf16x8 av = __builtin_bit_cast(bf16x8, acts[(mt * 16 + lr) * 32 + (c ^ lr)]);  // r & 15 == lr
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[mt], 0, 0, 0);
+        }
+      }
+  };
+
+  request(0);
+  fetch(wa, 0);
+  fetch(wb, 1);
+  const int rounds = nchunks / 3;
+  for (int it = 0; it < rounds; ++it) {  // three chunks: the roles of the weight registers come round
+    const int j = 3 * it;
+    chunk(j, wa, wc);
+    chunk(j + 1, wb, wa);
+    chunk(j + 2, wc, wb);
+  }
+  if (nchunks - 3 * rounds >= 1) chunk(3 * rounds, wa, wc);
+  if (nchunks - 3 * rounds == 2) chunk(3 * rounds + 1, wb, wa);
+
+  // ---- results: lane (lr, lg) holds out[m = mt * 16 + lr][n0 + 4 lg .. + 3]
+  floatx4* meet = reinterpret_cast<floatx4*>(tile_lds);  // [8 waves][MT][64], once the ring is done with
+  if constexpr (KW > 1 || GATED) {
+    __syncthreads();
+    if (kw > 0 || is_up) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) meet[(wave * MT + mt) * 64 + lane] = acc[mt];
+    }
+    __syncthreads();
+    if (kw > 0) return;
+    if constexpr (KW > 1) {  // the sums of the waves that shared this strip, in their order
+      if (!is_up) {
+#pragma unroll
+        for (int x = 1; x < KW; ++x)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt] += meet[((x * NS + strip) * MT + mt) * 64 + lane];
+      }
+    }
+    if (is_up) return;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + lr, n = n0 + 4 * lg;
+    floatx4 res = acc[mt];
+    if constexpr (GATED) {
+      floatx4 u = meet[((strip + OUT_STRIPS) * MT + mt) * 64 + lane];
+#pragma unroll
+      for (int x = 1; x < KW; ++x) u += meet[((x * NS + strip + OUT_STRIPS) * MT + mt) * 64 + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float g = rounded<OutT>(res[r]);
+        res[r] = g / (1.0f + expf(-g)) * rounded<OutT>(u[r]);
+      }
+    }
+    if (m >= M || n >= N) continue;
+    if constexpr (PARTIAL) {
+      store4<float>(partial + ((size_t)blockIdx.y * M + m) * N + n, res, min(4, N - n));
+    } else {
+      store4<OutT>(out + (size_t)m * N + n, res, min(4, N - n));
+    }
+  }
+}
+
+template <int MT, int NS>
+static int launch_tile(const void* a, const void* w, void* out, float* partial, int out_dtype, int M, int N, int K,
+                       int gated, int splits, hipStream_t stream) {
+  constexpr int TILE_WAVES = tile_waves(NS);
+  const size_t ring = (size_t)TILE_RING * MT * 16 * 32 * 16, meet = (size_t)TILE_WAVES * MT * 64 * 16;
+  const size_t shmem = ring > meet ? ring : meet;
+  const int k_per_split = K / (splits > 0 ? splits : 1);
+  const int per_tile = 16 * (gated ? NS / 2 : NS);
+  const dim3 grid((N + per_tile - 1) / per_tile, splits > 0 ? splits : 1);
+#define TILE_GO(GATEDV, PARTIALV, T)                                                                      \
+  do {                                                                                                    \
+    auto kernel = gemm_bf16_tile_kernel<MT, NS, GATEDV, PARTIALV, T>;                                     \
+    static bool raised = false;                                                                           \
+    if (shmem > (48u << 10) && !raised) {                                                                 \
+      if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,            \
+                              (int)shmem) != hipSuccess) return AS_LAUNCH_FAILED;                         \
+      raised = true;                                                                                      \
+    }                                                                                                     \
+    kernel<<<grid, TILE_WAVES * 64, shmem, stream>>>((const bf16*)a, (const bf16*)w, (T*)out, partial,    \
+                                                     M, N, K, k_per_split);                               \
+  } while (0)
+  if (splits > 0) TILE_GO(false, true, float);
+  else if (gated && out_dtype == DT_BF16) TILE_GO(true, false, bf16);
+  else if (!gated && out_dtype == DT_BF16) TILE_GO(false, false, bf16);
+  else if (!gated && out_dtype == DT_F32) TILE_GO(false, false, float);
+  else return AS_BAD_DTYPE;
+#undef TILE_GO
+  return launch_status();
+}
+
+// out[M, N] = a[M, K] @ w[N, K]^T for 1 <= M <= 64 and K % 256 == 0 through the tile kernel.
+//   gated != 0:  w is [2 N, K] (gate rows, then up rows), out[M, N] = silu(gate) * up, bf16.
+//   splits > 0:  K is cut into `splits` ranges (each a multiple of 256) and the fp32 sums of every
+//                range go to partial[splits, M, N]; `out` is not written.
+//   strips:      weight rows per workgroup / 16: 8, 6, 4 or 2 (0: 8).
+extern "C" int as_gemm_bf16_tile(const void* a, const void* w, void* out, float* partial, int out_dtype, int M,
+                                 int N, int K, int gated, int splits, int strips, hipStream_t stream) {
+  if (M <= 0) return AS_OK;
+  if (M > 64 || N <= 0 || K <= 0 || (K % TILE_KC) || splits < 0) return AS_BAD_SHAPE;
+  if (splits > 0 && (gated || !partial || (K % (splits * TILE_KC)))) return AS_BAD_SHAPE;
+  if (splits == 0 && !out) return AS_BAD_SHAPE;
+  if (strips == 0) strips = 8;
+  if (strips != 8 && strips != 6 && strips != 4 && strips != 2) return AS_BAD_SHAPE;
+  if ((unsigned long long)(gated ? 2 : 1) * N * K * 2ull > 0xf0000000ull) return AS_BAD_SHAPE;  // 32-bit byte offsets
+  const int MT = (M + 15) / 16;
+#define TILE_CASE(MTV, NSV) \
+  if (MT == MTV && strips == NSV) return launch_tile<MTV, NSV>(a, w, out, partial, out_dtype, M, N, K, gated, splits, stream)
+  TILE_CASE(1, 8); TILE_CASE(2, 8); TILE_CASE(3, 8); TILE_CASE(4, 8);
+  TILE_CASE(1, 6); TILE_CASE(2, 6); TILE_CASE(3, 6); TILE_CASE(4, 6);
+  TILE_CASE(1, 4); TILE_CASE(2, 4); TILE_CASE(3, 4); TILE_CASE(4, 4);
+  TILE_CASE(1, 2); TILE_CASE(2, 2); TILE_CASE(3, 2); TILE_CASE(4, 2);
+#undef TILE_CASE
+  return AS_BAD_SHAPE;
+}
+
 // strips: rows of w per workgroup / 16 in the streaming kernel (1, 2 or 4); 0 lets this
 // function choose, which for up to 16 rows and a K that fits is the persistent kernel (-1
 // asks for that one and fails where it cannot run).  Few strips (a small N) get 16 waves
@@ -529,7 +765,8 @@ extern "C" int as_gemm_bf16_skinny(const void* a, const void* w, void* out, int 
   }
   int S = strips;
   if (S == 0) S = 1;  // measured best at every size of interest; more strips only cost registers
-  if (MT > 2 && S > 1) S = 1;  // keeps the partial sums within LDS
+  if (S * MT > 8) S = 8 / MT;  // the partial sums of 8 waves stay within 64 KB of LDS
+  if (S == 3) S = 2;
   const bool wide = (N / (16 * S)) < 512 && MT <= 2 && S == 1;
 #define CASE(SV, MTV)                                                                               \
   if (S == SV && MT == MTV)                                                                         \
@@ -537,7 +774,7 @@ extern "C" int as_gemm_bf16_skinny(const void* a, const void* w, void* out, int 
                 : launch_skinny<SV, MTV, 8>(a, w, out, out_dtype, M, N, K, stream)
   CASE(1, 1); CASE(2, 1); CASE(4, 1);
   CASE(1, 2); CASE(2, 2); CASE(4, 2);
-  CASE(1, 3); CASE(1, 4);
+  CASE(1, 3); CASE(1, 4); CASE(2, 3); CASE(2, 4);
 #undef CASE
   return AS_BAD_SHAPE;
 }

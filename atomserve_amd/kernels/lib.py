@@ -20,6 +20,7 @@ SIGNATURES = {
     "as_embed_gather": ("elementwise", [P, I, P, P, I, I, I, F, P]),
     "as_logits_finish": ("elementwise", [P, c_longlong, F, F, P]),
     "as_rmsnorm": ("elementwise", [P, P, P, P, I, F, P, I, I, I, I, P]),
+    "as_rmsnorm_split": ("elementwise", [P, P, I, I, P, P, I, F, P, I, I, I, I, P]),
     "as_rope_table": ("elementwise", [P, P, P, I, I, P]),
     "as_qk_norm_rope_store": ("elementwise", [P, I, P, P, I, P, P, P, P, P, I, I, I, I, I, F, I, I, P]),
     "as_silu_mul": ("elementwise", [P, P, I, I, I, P]),
@@ -32,6 +33,7 @@ SIGNATURES = {
     "as_gemm_bf16_gated": ("gemm", [P, P, P, I, I, I, P]),
     "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, I, I, I, P]),
     "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, I, I, I, I, P]),
+    "as_gemm_bf16_tile": ("gemm", [P, P, P, P, I, I, I, I, I, I, I, P]),
     "as_blas_plan": ("blas", [I, I, I, I, c_size_t]),
     "as_blas_gemm": ("blas", [P, P, P, I, I, I, I, I, P, c_size_t, P]),
     "as_argmax": ("sampling", [P, P, I, I, P]),

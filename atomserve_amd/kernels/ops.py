@@ -63,9 +63,11 @@ def logits_finish(logits, scale: float = 1.0, softcap: float = 0.0) -> None:
     call("as_logits_finish", _ptr(logits), logits.numel(), float(scale), float(softcap), _stream())
 
 
-def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True) -> None:
+def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True, split_sums=None) -> None:
     """out[r] = norm(x[s] + delta[s]) * weight with s = rows[r] (or r); x fp32 [T, n] gets the
-    sum written back when `delta` is given and `update_x`.  out, delta: fp32|bf16."""
+    sum written back when `delta` is given and `update_x`.  out, delta: fp32|bf16.
+    split_sums: instead of `delta`, the fp32 partial sums [splits, T, n] of the product that makes it
+    (`gemm_split`); they are added up and rounded to out's dtype as the product would have been."""
     _check(x, "x", F32, (None, None))
     T, n = x.shape
     _check(weight, "weight", (F32, BF16), (n,))
@@ -78,6 +80,13 @@ def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True) -> None:
         _check(delta, "delta", out.dtype, (T, n))
     if out.dtype == F32 and weight.dtype != F32:
         raise KernelError("fp32 norm needs an fp32 weight")
+    if split_sums is not None:
+        if delta is not None:
+            raise KernelError("a pending sum comes as one tensor or as partial sums, not both")
+        _check(split_sums, "split_sums", F32, (None, T, n))
+        call("as_rmsnorm_split", _ptr(x), _ptr(split_sums), split_sums.shape[0], T, _ptr(rows), _ptr(weight),
+             _DT[weight.dtype], float(eps), _ptr(out), _DT[out.dtype], n_out, n, int(bool(update_x)), _stream())  # fmt: skip
+        return
     call("as_rmsnorm", _ptr(x), _ptr(delta), _ptr(rows), _ptr(weight), _DT[weight.dtype], float(eps), _ptr(out),
          _DT[out.dtype], n_out, n, int(bool(update_x)), _stream())  # fmt: skip
 
@@ -517,6 +526,45 @@ def _fastest_of(trial) -> int:
     return best
 
 
+# ---- 17 to 64 rows: tiles of weight rows with the activations staged in LDS ---------------------
+TILE_MAX_ROWS = 64
+TILE_CHUNK = 256  # K comes in chunks of this many
+
+
+def _tile_rows(rows: int, k: int, dtype) -> bool:
+    return dtype == BF16 and SKINNY_MAX_ROWS < rows <= TILE_MAX_ROWS and k % TILE_CHUNK == 0
+
+
+def gemm_split_plan(rows: int, n: int, k: int, dtype):
+    """(strips, splits) of `gemm_split` for a product of these sizes, or None where it has no kernel:
+    tiles of 64 weight rows, and K cut into as many ranges (of whole chunks) as fill the compute
+    units with those tiles."""
+    if not _tile_rows(rows, k, dtype) or n % 4:
+        return None
+    strips = 4
+    tiles = -(-n // (16 * strips))
+    chunks = k // TILE_CHUNK
+    want = max(1, compute_units() // tiles)
+    splits = max(d for d in range(1, chunks + 1) if chunks % d == 0 and d <= want)
+    return strips, splits
+
+
+def gemm_split(a, w, plan=None):
+    """The fp32 partial sums [splits, M, N] of a[M, K] @ w[N, K]^T with K cut into `splits` ranges;
+    whoever takes them adds them up (`rmsnorm(..., split_sums=)`).  bf16, 17 to 64 rows."""
+    _check(a, "a", BF16, (None, None))
+    M, K = a.shape
+    _check(w, "w", BF16, (None, K))
+    N = w.shape[0]
+    plan = plan or gemm_split_plan(M, N, K, a.dtype)
+    if plan is None:
+        raise KernelError(f"gemm_split: {M} rows, {K} -> {N} have no kernel")
+    strips, splits = plan
+    sums = torch.empty((splits, M, N), dtype=F32, device=a.device)
+    call("as_gemm_bf16_tile", _ptr(a), _ptr(w), 0, _ptr(sums), _DT[F32], M, N, K, 0, splits, strips, _stream())
+    return sums
+
+
 GATED_MAX_K = 6144  # the widest input the fused product-and-activation kernel keeps in registers
 
 
@@ -542,6 +590,9 @@ def gemm_silu_mul(a, w, out) -> None:
         return
     if a.dtype == BF16 and (_few_rows(M, K, inter, GATED_MAX_K) or _gated_two_tiles(M, K)):
         call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), M, inter, K, _stream())
+        return
+    if _tile_rows(M, K, a.dtype):
+        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0, 8, _stream())
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
     gemm(a, w, gate_up)

@@ -12,7 +12,7 @@ run's cache computes q alone and stores nothing.
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import Mixer, PagedCacheRequest, PendingNorm, WeightDecl, build, register
+from atomserve_amd.parts.base import Mixer, PagedCacheRequest, PendingNorm, SplitSums, WeightDecl, build, register
 
 # Rows with at most SHORT_ROW new tokens are attended as that many single queries
 # (reference atomserve/runner.py:31-34); longer rows go through the prefill kernel in work items of
@@ -98,6 +98,10 @@ class Attention(Mixer):
             link = next_norm.absorb(out.view(T, H * D), self.o_weight, residual)
             if link is not None:
                 return link
+            if next_norm.takes_split_sums:
+                plan = ops.gemm_split_plan(T, s.hidden_size, out.view(T, H * D).shape[1], env.dtype)
+                if plan is not None:
+                    return SplitSums(ops.gemm_split(out.view(T, H * D), self.o_weight, plan))
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=device)
         ops.gemm(out.view(T, H * D), self.o_weight, y)
         return y

@@ -109,12 +109,22 @@ class PendingNorm:
         return False
 
 
+class SplitSums:
+    """The output of a part's last matrix product as fp32 partial sums [splits, T, hidden] over
+    ranges of K, still to be added up and into the stream: a norm that says `takes_split_sums`
+    does both in its own kernel."""
+
+    def __init__(self, sums: torch.Tensor):
+        self.sums = sums
+
+
 class Mixer(Part):
     # Two optional shortcuts an arrangement may take with a part that declares them:
     # takes_pending_norm: `h` may arrive as a PendingNorm instead of normalised rows;
     # adds_to_residual: forward accepts `residual=` (the fp32 stream) and `next_norm=` (the norm
     #   that follows); where its last product can add into the stream and leave that norm
-    #   pending (`Norm.absorb`), it returns the PendingNorm instead of its output.
+    #   pending (`Norm.absorb`), it returns the PendingNorm instead of its output; where that norm
+    #   `takes_split_sums` it may return its output as `SplitSums`.
     takes_pending_norm = False
     adds_to_residual = False
 
@@ -141,6 +151,8 @@ class FeedForward(Part):
 
 
 class Norm(Part):
+    takes_split_sums = False  # whether `forward` accepts a SplitSums as `delta`
+
     def forward(self, x, delta=None, rows=None, update_residual=True) -> torch.Tensor:
         raise NotImplementedError
 

@@ -4,7 +4,7 @@ one matrix (reference atomserve/model.py:339-360)."""
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import FeedForward, PendingNorm, WeightDecl, register
+from atomserve_amd.parts.base import FeedForward, PendingNorm, SplitSums, WeightDecl, register
 
 
 class GatedMLP(FeedForward):
@@ -35,6 +35,10 @@ class GatedMLP(FeedForward):
             link = next_norm.absorb(act, self.down_weight, residual)
             if link is not None:
                 return link
+            if next_norm.takes_split_sums:
+                plan = ops.gemm_split_plan(T, s.hidden_size, act.shape[1], env.dtype)
+                if plan is not None:
+                    return SplitSums(ops.gemm_split(act, self.down_weight, plan))
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=device)
         ops.gemm(act, self.down_weight, y)
         return y

@@ -6,7 +6,7 @@ pre-norm layer is fused into the same kernel: the fp32 residual stream `x` recei
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import Norm, PendingNorm, WeightDecl, register
+from atomserve_amd.parts.base import Norm, PendingNorm, SplitSums, WeightDecl, register
 
 
 class PendingRMSNorm(PendingNorm):
@@ -29,6 +29,7 @@ class PendingRMSNorm(PendingNorm):
 
 class RMSNorm(Norm):
     capturable = True
+    takes_split_sums = True
 
     def weight_decls(self) -> dict:
         return {"weight": WeightDecl((self.spec.size,), role="vector")}
@@ -47,11 +48,15 @@ class RMSNorm(Norm):
         return PendingRMSNorm(self, x, scaled, ssq)
 
     def forward(self, x, delta=None, rows=None, update_residual=True) -> torch.Tensor:
-        """x: fp32 [T, size] residual stream.  delta: pending sum in the compute dtype, or None.
+        """x: fp32 [T, size] residual stream.  delta: pending sum in the compute dtype (or as the
+        partial sums of the product that makes it, `SplitSums`), or None.
         rows: int32 row selection, or None for all rows.  Returns [rows, size], compute dtype."""
         n_out = x.shape[0] if rows is None else rows.shape[0]
         out = torch.empty((n_out, self.spec.size), dtype=self.env.dtype, device=x.device)
-        ops.rmsnorm(x, self.weight, self.spec.eps, out, delta=delta, rows=rows, update_x=update_residual)
+        if isinstance(delta, SplitSums):
+            ops.rmsnorm(x, self.weight, self.spec.eps, out, rows=rows, update_x=update_residual, split_sums=delta.sums)
+        else:
+            ops.rmsnorm(x, self.weight, self.spec.eps, out, delta=delta, rows=rows, update_x=update_residual)
         return out
 
 

@@ -323,11 +323,11 @@ def test_gemm_silu_mul_bf16(ops, M, I, K):
     two = torch.empty(M, I, dtype=BF16, device=DEV)
     ops.silu_mul(gate_up, two)
     assert close_bf16(gate_up, pk.gemm(a, w), scale=1.0)
-    if M <= 16 or M > 32 or ops._few_rows(M, K, 2 * I):
+    if M <= 16 or ops._few_rows(M, K, 2 * I) or (M > 32 and not ops._tile_rows(M, K, BF16)):
         assert torch.equal(out, two)  # the same products, whichever kernels made them
         assert close_bf16(out, pk.silu_mul(gate_up))
     else:
-        # 17 to 32 wide rows: the gated kernel is this package's, the plain product the library's; their sums
+        # 17 to 64 wide rows: the gated kernel is this package's, the plain product the library's; their sums
         # differ in the last bit now and then, and the activation carries that on
         assert (out != two).float().mean() < 0.05
         assert torch.allclose(out.float(), pk.silu_mul(pk.gemm(a, w).to(BF16)).float(), atol=2e-2, rtol=2e-2)
@@ -863,3 +863,55 @@ def test_sampling_is_seeded_per_request_and_mixes_greedy_rows(ops):
         crowd.append(int(out[1]))
         assert int(out[2]) == int(logits[2].argmax())  # the greedy row is its argmax
     assert alone == crowd and len(set(alone)) > 1
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 96, 256), (33, 1000, 512), (64, 4096, 1024), (48, 520, 768), (20, 64, 3072), (64, 12, 256)])
+def test_products_of_17_to_64_rows_in_tiles(ops, M, N, K):
+    """The tile kernel behind `gemm_silu_mul` and `gemm_split`: every tile width (8, 6, 4 and 2 strips),
+    plain, gated and with K cut into ranges, against the matrix product in float64; rows and columns that
+    do not fill the last tile, chunk counts that are no multiple of three."""
+    from atomserve_amd.kernels.lib import call
+
+    torch.manual_seed(M + N)
+    a = (torch.randn(M, K, device=DEV) * 0.5).to(BF16)
+    w = (torch.randn(2 * N, K, device=DEV) * 0.1).to(BF16)
+    stream = torch.cuda.current_stream().cuda_stream
+    ref = a.double() @ w.double().T
+    gated_ref = (lambda g: torch.nn.functional.silu(g[:, :N]) * g[:, N:])(ref.to(BF16).double())
+    chunks = K // 256
+    for strips in (8, 6, 4, 2):
+        out = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
+        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), out.data_ptr(), 0, 1, M, N, K, 0, 0, strips, stream)
+        assert close_bf16(out, ref[:, :N]), f"plain, {strips} strips"
+        out32 = torch.full((M, N), float("nan"), dtype=F32, device=DEV)
+        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), out32.data_ptr(), 0, 0, M, N, K, 0, 0, strips, stream)
+        assert torch.allclose(out32.double(), ref[:, :N], atol=1e-3, rtol=1e-4)
+        out.fill_(float("nan"))
+        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), out.data_ptr(), 0, 1, M, N, K, 1, 0, strips, stream)
+        # a sum that rounds to the neighbouring bfloat16 moves the activation by a step of its input
+        assert torch.allclose(out.double(), gated_ref, atol=2e-2, rtol=2e-2), f"gated, {strips} strips"
+        for splits in {1, chunks, max(1, chunks // 2)}:
+            if chunks % splits:
+                continue
+            sums = torch.full((splits, M, N), float("nan"), dtype=F32, device=DEV)
+            call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), 0, sums.data_ptr(), 0, M, N, K, 0, splits, strips, stream)
+            assert torch.allclose(sums.double().sum(0), ref[:, :N], atol=1e-3, rtol=1e-4), f"{splits} ranges, {strips} strips"
+    # through the wrappers: the gated product, and split sums taken in by the norm
+    act = torch.empty(M, N, dtype=BF16, device=DEV)
+    ops.gemm_silu_mul(a, w, act)
+    assert torch.allclose(act.double(), gated_ref, atol=2e-2, rtol=2e-2)
+    if N % 4 == 0:
+        sums = ops.gemm_split(a, w[:N].contiguous())
+        x = torch.randn(M, N, device=DEV)
+        gain = (torch.randn(N, device=DEV) + 1).to(BF16)
+        x1, x2 = x.clone(), x.clone()
+        out1, out2 = torch.empty(M, N, dtype=BF16, device=DEV), torch.empty(M, N, dtype=BF16, device=DEV)
+        ops.rmsnorm(x1, gain, 1e-5, out1, split_sums=sums)
+        delta = sums.sum(0).to(BF16)
+        ops.rmsnorm(x2, gain, 1e-5, out2, delta=delta)
+        assert torch.allclose(x1, x2, atol=1e-6) and close_bf16(out1, out2.double())
+        rows = i32([M - 1, 0, 3])
+        sel = torch.empty(3, N, dtype=BF16, device=DEV)
+        x3 = x.clone()
+        ops.rmsnorm(x3, gain, 1e-5, sel, rows=rows, update_x=False, split_sums=sums)
+        assert torch.equal(x3, x) and close_bf16(sel, out2[[M - 1, 0, 3]].double())
