@@ -583,11 +583,16 @@ __global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(con
     const int slot = i * NT + tid, r = slot >> 5, c = (slot & 31) ^ (r & 15);
     a_off[i] = slot < SLOTS ? ((unsigned)min(r, M - 1) * (unsigned)K + k0 + c * 8) * 2u : BEYOND;
   }
+  // Workgroups start at different chunks of K and wrap round: side by side they would all ask for
+  // the same 512 bytes of every weight row at the same time, which are the same few memory channels.
+  const int turn = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)max(nchunks, 1));
+  auto where = [&](int j) { const int at = j + turn; return at >= nchunks ? at - nchunks : at; };
   auto request = [&](int j) {
+    const int at = where(j);
 #pragma unroll
     for (int i = 0; i < COPIES; ++i)
       held[i] = __builtin_amdgcn_raw_buffer_load_b128(
-          a_buf, (j < nchunks && a_off[i] != BEYOND) ? a_off[i] + j * (TILE_KC * 2) : BEYOND, 0, 0);
+          a_buf, (j < nchunks && a_off[i] != BEYOND) ? a_off[i] + at * (TILE_KC * 2) : BEYOND, 0, 0);
   };
   auto deposit = [&](int j) {
     u32x4_t* dst = tile_lds + (j % TILE_RING) * SLOTS + tid;
@@ -599,7 +604,7 @@ __global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(con
   // roles rotate with the chunks (copying one set into another would wait for the newest loads).
   u32x4_t wa[STEPS][2], wb[STEPS][2], wc[STEPS][2];
   auto fetch = [&](u32x4_t (&into)[STEPS][2], int j) {
-    const unsigned base = j < nchunks ? w_off + j * (TILE_KC * 2) : BEYOND;
+    const unsigned base = j < nchunks ? w_off + where(j) * (TILE_KC * 2) : BEYOND;
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
       const unsigned at = j < nchunks ? base + (kw + i * KW) * 128 : BEYOND;

@@ -535,6 +535,17 @@ def _tile_rows(rows: int, k: int, dtype) -> bool:
     return dtype == BF16 and SKINNY_MAX_ROWS < rows <= TILE_MAX_ROWS and k % TILE_CHUNK == 0
 
 
+def _gated_tile_strips(rows: int, outputs: int) -> int:
+    """Strips of 16 weight rows (gate and up together) per workgroup of the gated tile kernel: a
+    workgroup loads 16 rows of weights per strip and `rows` rows of activations, and the workgroups
+    run in rounds of one per compute unit; the width with the least to load on the longest path."""
+    def cost(strips):
+        tiles = -(-outputs // (8 * strips))
+        return -(-tiles // compute_units()) * (16 * strips + rows)
+
+    return min((8, 6, 4, 2), key=cost)
+
+
 def gemm_split_plan(rows: int, n: int, k: int, dtype):
     """(strips, splits) of `gemm_split` for a product of these sizes, or None where it has no kernel:
     tiles of 64 weight rows, and K cut into as many ranges (of whole chunks) as fill the compute
@@ -592,7 +603,8 @@ def gemm_silu_mul(a, w, out) -> None:
         call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _ptr(out), M, inter, K, _stream())
         return
     if _tile_rows(M, K, a.dtype):
-        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0, 8, _stream())
+        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0,
+             _gated_tile_strips(M, inter), _stream())  # fmt: skip
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
     gemm(a, w, gate_up)
