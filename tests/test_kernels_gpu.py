@@ -293,7 +293,8 @@ def test_gemm_fp32_rows_do_not_depend_on_the_batch(ops):
                                    (16, 4096, 4096), (12, 8200, 4096), (9, 16000, 2048), (3, 40, 200), (16, 24, 8),
                                    (4, 1040, 5120), (7, 520, 6144), (2, 100, 2560), (11, 4100, 3072), (8, 512, 12288),
                                    (13, 300, 6152), (17, 300, 4096), (32, 6144, 1024), (25, 1000, 1000),
-                                   (31, 520, 3072), (20, 64, 4096), (32, 300, 24), (32, 6144, 4096)])  # fmt: skip
+                                   (31, 520, 3072), (20, 64, 4096), (32, 300, 24), (32, 6144, 4096), (8, 6150, 4096), (1, 10240, 2048),
+                                   (24, 6147, 1024)])  # fmt: skip
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(8)
     a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
@@ -448,7 +449,7 @@ def test_gemm_link_bf16(ops, M, N, K):
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 6144, 4096), (9, 700, 2048),
                                    (3, 40, 200), (16, 24, 8), (7, 264, 3072), (2, 130, 5120), (32, 6144, 1024),
-                                   (17, 1030, 2048), (26, 40, 200), (31, 264, 2048)])  # fmt: skip
+                                   (17, 1030, 2048), (26, 40, 200), (31, 264, 2048), (6, 6148, 4096), (20, 6144, 2048)])  # fmt: skip
 def test_gemm_scaled_bf16(ops, M, N, K, gated):
     """The product that finishes a pending norm: x * gain arrives rounded to bf16, 1 / rms comes
     from the sums of squares and multiplies the fp32 sums.  That input times the plain 1 / rms is
