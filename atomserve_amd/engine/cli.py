@@ -98,6 +98,10 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--presence-penalty", type=float, default=0.0, help="subtracted from logits of generated tokens")
     p.add_argument("--seed", type=int, default=None, help="fixed seed for reproducible sampling")
     p.add_argument("--ignore-eos", action="store_true", help="keep generating past end-of-sequence")
+    p.add_argument("--fixed-products", action="store_true",
+                   help="always take the library's first candidate for its matrix products instead of timing them at "
+                        "start-up: bfloat16 results are then the same from run to run (a little slower at 17 to 64 "
+                        "requests and for prompts)")  # fmt: skip
     p.add_argument("--version", action="version", version=f"%(prog)s {__version__}")
     return p
 
@@ -184,12 +188,16 @@ def main(argv=None) -> int:
     if args.kv_mem_gb * 2**30 // block_bytes > 2**31 // args.block_size:  # slots are 32-bit integers
         args.kv_mem_gb = (2**31 // args.block_size) * block_bytes / 2**30
     engine_config = engine_config_for(args, block_bytes, model.plan.max_positions)
+    from atomserve_amd.kernels import ops
+
+    ops.fix_library_choices(args.fixed_products)
     engine = create_engine(model, engine_config, eos_ids(model_dir), seed=args.seed)
     engine.generate([[0]], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))  # compile and warm up
     engine.warm_up()  # and capture the decode steps of every batch size now, not at their first use
     print(
         f"Ready in {time.perf_counter() - start:.1f}s. KV cache: "
-        f"{engine_config.num_blocks * engine_config.block_size:,} tokens, context up to {engine_config.max_model_len:,}.",
+        f"{engine_config.num_blocks * engine_config.block_size:,} tokens, context up to {engine_config.max_model_len:,}; "
+        f"captured decode steps hold {engine.stats().get('graph_bytes', 0) / 2**20:,.0f} MiB.",
         file=sys.stderr, flush=True,
     )  # fmt: skip
 
