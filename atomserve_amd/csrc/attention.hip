@@ -732,42 +732,61 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
 
   // ---- this wave's share of the copies: of every 32-key step, waves 0 and 1 bring the keys
   // (half of the 16-byte chunks of all 32 rows each), waves 2 and 3 the values of keys 0-15 and
-  // 16-31.  A 16-key piece that would start beyond the last key repeats the last one (finite
-  // numbers; its scores are masked).
+  // 16-31.
   const int kb0 = (wg_lo / 32) * 32;
   const int nsteps = (wg_last - kb0) / 32 + 1;
   const int last_piece = (wg_last / 16) * 16;
-  auto page_of = [&](int step, int piece) { return table[min(kb0 + 32 * step + 16 * piece, last_piece) / bs]; };
-  int page_next[2] = {page_of(0, 0), page_of(0, 1)};
-  auto issue = [&](int step) {
-    size_t base[2];
-    int off0[2];
+  // Where the 16-key pieces lie in memory is worked out 64 pieces at a time, one piece per lane
+  // (its page from the block table, asked for one batch of 64 ahead), and a step reads the two
+  // it copies out of those lanes.  Done by the scalar unit for every step instead, the divisions
+  // by the page size and the 64-bit products took a fifth of the kernel's time: that unit is
+  // shared by all waves of the compute unit.  A piece that would start beyond the last key
+  // repeats the last one (finite numbers; its scores are masked).
+  unsigned long long k_at = 0, v_at = 0;  // byte offsets of this lane's piece in k_pages and v_pages
+  auto entry_of = [&](int piece) { return min(kb0 + 16 * piece, last_piece) / bs; };
+  int page_ahead = table[entry_of(lane)];
+  auto locate = [&](int batch) {  // pieces 64 batch .. 64 batch + 63
+    const int piece = 64 * batch + lane, key = min(kb0 + 16 * piece, last_piece);
+    const unsigned long long row = (unsigned long long)((unsigned)page_ahead * KV + kvh) * bs;
+    k_at = (row + key % bs) * (D * 2);
+    v_at = (row * D + key % bs) * 2;
+    page_ahead = table[entry_of(piece + 64)];
+  };
+  auto at = [&](unsigned long long offsets, int piece) {
+    const unsigned lo = __builtin_amdgcn_readlane((unsigned)offsets, piece & 63);
+    const unsigned hi = __builtin_amdgcn_readlane((unsigned)(offsets >> 32), piece & 63);
+    return ((unsigned long long)hi << 32) | lo;
+  };
+  // what of a copy's address belongs to the lane, in bytes
+  int lane_at[DC];
+  if (wave >= 2) {
 #pragma unroll
-    for (int pc = 0; pc < 2; ++pc) {
-      off0[pc] = min(kb0 + 32 * step + 16 * pc, last_piece) % bs;
-      base[pc] = ((size_t)page_next[pc] * KV + kvh) * bs * D;
-      page_next[pc] = page_of(step + 1, pc);  // scalar loads with a whole step to arrive
+    for (int i = 0; i < DC; ++i) {  // values: slot = h * D + d holds keys 8h .. 8h+7 of coordinate d
+      const int slot = i * 64 + lane, h = slot / D, d = slot % D;
+      lane_at[i] = (d * bs + h * 8) * 2;
     }
+  } else {
+    // keys: slot = chunk * 32 + t holds coordinates 8 chunk .. + 7 of the key that row t of the
+    // step's two score tiles stands for (see PF_KEY_OF_ROW)
+    const int t = lane & 31, key = PF_KEY_OF_ROW(t >> 4, t & 15);
+    lane_at[0] = ((key & 15) * D + (wave * (2 * DC) + (lane >> 5)) * 8) * 2;  // the further chunks: + 32 bytes each
+  }
+  const bool second_piece = PF_KEY_OF_ROW((lane & 31) >> 4, lane & 15) >> 4;
+  auto issue = [&](int step) {
+    if ((step & 31) == 0) locate(step >> 5);
     if (wave >= 2) {
-      // values of one piece: slot = h * D + d holds keys 8h .. 8h+7 of coordinate d
-      const int pc = wave - 2;
-      u32x4_t* dst = &lds[step % PF_STAGES][2 + pc][0];
-#pragma unroll
-      for (int i = 0; i < DC; ++i) {
-        const int slot = i * 64 + lane, h = slot / D, d = slot % D;
-        __builtin_amdgcn_global_load_lds((global_ptr_t)(v_pages + base[pc] + (size_t)d * bs + off0[pc] + h * 8),
-                                         (lds_ptr_t)(dst + i * 64), 16, 0, 0);
-      }
-    } else {
-      // keys: slot = chunk * 32 + t holds coordinates 8 chunk .. + 7 of the key that row t of the
-      // step's two score tiles stands for (see PF_KEY_OF_ROW)
-      u32x4_t* dst = &lds[step % PF_STAGES][0][0] + wave * (DC * 64);
-      const int t = lane & 31, key = PF_KEY_OF_ROW(t >> 4, t & 15), pc = key >> 4;
-      const bf16* src = k_pages + (pc ? base[1] : base[0]) + (size_t)((pc ? off0[1] : off0[0]) + (key & 15)) * D +
-                        (wave * (2 * DC) + (lane >> 5)) * 8;
+      const char* src = reinterpret_cast<const char*>(v_pages) + at(v_at, 2 * step + wave - 2);
+      u32x4_t* dst = &lds[step % PF_STAGES][wave][0];
 #pragma unroll
       for (int i = 0; i < DC; ++i)
-        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + i * 16), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + lane_at[i]), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
+    } else {
+      const unsigned long long first = at(k_at, 2 * step), second = at(k_at, 2 * step + 1);
+      const char* src = reinterpret_cast<const char*>(k_pages) + (second_piece ? second : first) + lane_at[0];
+      u32x4_t* dst = &lds[step % PF_STAGES][0][0] + wave * (DC * 64);
+#pragma unroll
+      for (int i = 0; i < DC; ++i)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(src + i * 32), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
     }
   };
   const int nrounds = (nsteps + 1) / 2;

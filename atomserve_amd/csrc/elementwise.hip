@@ -415,13 +415,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_bf16x8_kernel(
     Gain8<W>::load(w + 8 * l, ga);
     Gain8<W>::load(w + half + 8 * l, gb);
   }
+  // the angles of this lane's eight pairs: 64 contiguous bytes, four loads
+  float4 turn[4];
+  if (cs) {
+    const float4* cs4 = reinterpret_cast<const float4*>(cs + t * half + 8 * l);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) turn[j] = cs4[j];
+  }
   bf16x8 oa, ob;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     float a = (float)a8[j] * inv, b = (float)b8[j] * inv;
     if (w) { a *= ga[j]; b *= gb[j]; }
     float c = 1.f, sn = 0.f;
-    if (cs) { const float2 v = cs[t * half + 8 * l + j]; c = v.x; sn = v.y; }
+    if (cs) { c = (j & 1) ? turn[j >> 1].z : turn[j >> 1].x; sn = (j & 1) ? turn[j >> 1].w : turn[j >> 1].y; }
     oa[j] = (bf16)(a * c - b * sn);
     ob[j] = (bf16)(b * c + a * sn);
     if (is_k) { oa[j] = finite_or_zero((bf16)oa[j]); ob[j] = finite_or_zero((bf16)ob[j]); }
