@@ -253,16 +253,38 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-// The keys and values of one step (32 keys = two tiles of 16) of one kv head, as the MFMA
-// operands of this lane: keys as rows of A (16 bytes of each key's head), values as the
-// transposed page gives them (4 keys of one coordinate).  A tile that starts at or beyond
-// `end` is not read and counts as zeros.  Loading the next step before computing the current
-// one keeps memory busy while the matrix cores work.
+// Which of a step's 32 keys row `row` of its score tile `tile` (0, 1) stands for.  Rows 4g..4g+3
+// of both tiles are what lane group g holds after the score product, and they are keys
+// 8g .. 8g+7: eight neighbours, whose values are one 16-byte piece of a transposed page.
+#define KEY_OF_ROW(tile, row) (8 * ((row) >> 2) + ((row) & 3) + 4 * (tile))
+
+// Sums and maxima over the four lanes that share `lane % 16` (lane ^ 16, lane ^ 32) without a
+// trip through LDS: v_permlane16_swap / v_permlane32_swap exchange rows of 16 lanes between
+// two registers.  With both operands equal to x, the results hold (rows 0 0 2 2, rows 1 1 3 3)
+// and (rows 0 1 0 1, rows 2 3 2 3) of x.
+__device__ __forceinline__ float quad_rows_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// The keys and values of one step (32 keys, two 16-key pieces of pages) of one kv head, as the
+// MFMA operands of this lane: keys as rows of A (16 bytes of the head of key KEY_OF_ROW(tile,
+// lane % 16)), values as the transposed page gives them (the lane group's 8 keys of one
+// coordinate: 16 bytes).  A piece that starts at or beyond `end` is not read and counts as zeros.
+// Loading the next step before computing the current one keeps memory busy while the matrix
+// cores work.
 template <int DC>
 struct KVStep {
   bf16x8_t k[2][DC];
-  bf16x4_t v[2][2 * DC];
-  bool live[2];
+  bf16x8_t v[2 * DC];
 };
 
 template <int DC>
@@ -270,25 +292,33 @@ __device__ __forceinline__ void load_kv_step(KVStep<DC>& st, const bf16* __restr
                                              const bf16* __restrict__ v_pages, const int* __restrict__ table,
                                              int kb, int end, int KV, int kvh, int bs, int col, int grp) {
   constexpr int D = DC * 32, DT = DC * 2;
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  size_t head[2];
+  int off0[2];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) {
-    const int key0 = kb + 16 * tt;
-    st.live[tt] = key0 < end;
-    if (st.live[tt]) {
-      const int page = table[key0 / bs], off0 = key0 % bs;
-      const size_t head = ((size_t)page * KV + kvh) * bs * D;
-      const bf16* krow = k_pages + head + (size_t)(off0 + col) * D + grp * 8;
+  for (int pc = 0; pc < 2; ++pc) {  // uniform over the wave
+    const int key0 = kb + 16 * pc;
+    const int page = key0 < end ? table[key0 / bs] : 0;
+    head[pc] = ((size_t)page * KV + kvh) * bs * D;
+    off0[pc] = key0 % bs;
+  }
+  {  // keys: rows 0-7 of both tiles lie in the first piece, rows 8-15 in the second
+    const int pc = col >> 3;
+    const bool live = kb + 16 * pc < end;
+    const bf16* krow = k_pages + (pc ? head[1] : head[0]) + (size_t)((pc ? off0[1] : off0[0]) + (KEY_OF_ROW(0, col) & 15)) * D + grp * 8;
 #pragma unroll
-      for (int c = 0; c < DC; ++c) st.k[tt][c] = *reinterpret_cast<const bf16x8_t*>(krow + c * 32);
-      const bf16* vcol = v_pages + head + off0 + 4 * grp + (size_t)col * bs;
+    for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) st.v[tt][dt] = *reinterpret_cast<const bf16x4_t*>(vcol + (size_t)dt * 16 * bs);
-    } else {
+      for (int c = 0; c < DC; ++c)
+        st.k[tt][c] = live ? *reinterpret_cast<const bf16x8_t*>(krow + (size_t)tt * 4 * D + c * 32) : zero;
+  }
+  {  // values: keys 8 grp .. 8 grp + 7 of coordinates col, col + 16, ...
+    const int pc = grp >> 1;
+    const bool live = kb + 16 * pc < end;
+    const bf16* vcol = v_pages + (pc ? head[1] : head[0]) + (pc ? off0[1] : off0[0]) + 8 * (grp & 1) + (size_t)col * bs;
 #pragma unroll
-      for (int c = 0; c < DC; ++c) st.k[tt][c] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) st.v[tt][dt] = bf16x4_t{0, 0, 0, 0};
-    }
+    for (int dt = 0; dt < DT; ++dt)
+      st.v[dt] = live ? *reinterpret_cast<const bf16x8_t*>(vcol + (size_t)dt * 16 * bs) : zero;
   }
 }
 
@@ -482,21 +512,22 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 128, k1, KV, kvh, bs, col, grp);
     if constexpr (FRESH != 0) {
       if (fresh_here && pos >= kb && pos < kb + 32) {  // this wave's step holds the token itself: take it from LDS
-        const int at = pos - kb;
+        const int at = pos - kb;  // = KEY_OF_ROW(tile, row) for
+        const int tile = (at >> 2) & 1, row = 4 * (at >> 3) + (at & 3);
+        if (col == row) {
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-          if ((at >> 4) != tt) continue;
-          if (col == (at & 15)) {
+          for (int tt = 0; tt < 2; ++tt)
+            if (tt == tile) {
 #pragma unroll
-            for (int c = 0; c < DC; ++c) cur.k[tt][c] = *reinterpret_cast<const bf16x8_t*>(&fresh_kv[0][c * 32 + grp * 8]);
-          }
-          if (grp == ((at & 15) >> 2)) {
+              for (int c = 0; c < DC; ++c) cur.k[tt][c] = *reinterpret_cast<const bf16x8_t*>(&fresh_kv[0][c * 32 + grp * 8]);
+            }
+        }
+        if (grp == (at >> 3)) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+          for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (r == (at & 3)) cur.v[tt][dt][r] = fresh_kv[1][dt * 16 + col];
-          }
+            for (int j = 0; j < 8; ++j)
+              if (j == (at & 7)) cur.v[dt][j] = fresh_kv[1][dt * 16 + col];
         }
       }
     }
@@ -514,13 +545,12 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int key = kb + 16 * tt + 4 * grp + r;
-        const bool seen = cur.live[tt] && key >= k0 && key < k1;
+        const int key = kb + KEY_OF_ROW(tt, 4 * grp + r);
+        const bool seen = key >= k0 && key < k1;
         s[tt][r] = seen ? s[tt][r] * scale : NEG_INF;
         mx = fmaxf(mx, s[tt][r]);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    mx = quad_rows_max(mx);
     const float mn = fmaxf(m, mx);
     float alpha = 1.f, rs = 0.f;
     bf16x8_t pop;
@@ -539,19 +569,12 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         }
       m = mn;
     }
-    rs += __shfl_xor(rs, 16, WAVE);
-    rs += __shfl_xor(rs, 32, WAVE);
-    l = l * alpha + rs;
+    l = l * alpha + quad_rows_sum(rs);
     // ---- weighted values
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      bf16x8_t vop;
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) vop[tt * 4 + r] = cur.v[tt][dt][r];
       o[dt] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.v[dt], pop, o[dt], 0, 0, 0);
     }
     if (more) cur = nxt;
   }
@@ -616,34 +639,14 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 // A load instruction fills 64 consecutive slots (slot = first + lane); which 16 bytes of
 // memory a lane fetches is free, which is how the key layout comes about.
 // A query at position p sees keys lo..p by absolute position, wherever the row starts.
-// Sums and maxima over the four lanes that share `lane % 16` (lane ^ 16, lane ^ 32) without a
-// trip through LDS: v_permlane16_swap / v_permlane32_swap exchange rows of 16 lanes between
-// two registers.  With both operands equal to x, the results hold (rows 0 0 2 2, rows 1 1 3 3)
-// and (rows 0 1 0 1, rows 2 3 2 3) of x.
 // max(a, b, c) as the one instruction it is; NaN operands lose, as with fmaxf.
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
-__device__ __forceinline__ float quad_rows_max(float v) {
-  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-__device__ __forceinline__ float quad_rows_sum(float v) {
-  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
 
 #define PF_STAGES 4
-// Which of a step's 32 keys row `row` of its score tile `tile` (0, 1) stands for.  Rows 4g..4g+3
-// of both tiles are what lane group g holds after the score product, and they are keys
-// 8g .. 8g+7: eight neighbours, whose values are one 16-byte piece of a transposed page.
-#define PF_KEY_OF_ROW(tile, row) (8 * ((row) >> 2) + ((row) & 3) + 4 * (tile))
 // s_waitcnt that only constrains the vector-memory counter (vmcnt: bits 3:0 and 15:14)
 #define PF_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
 
@@ -767,11 +770,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     }
   } else {
     // keys: slot = chunk * 32 + t holds coordinates 8 chunk .. + 7 of the key that row t of the
-    // step's two score tiles stands for (see PF_KEY_OF_ROW)
-    const int t = lane & 31, key = PF_KEY_OF_ROW(t >> 4, t & 15);
+    // step's two score tiles stands for (see KEY_OF_ROW)
+    const int t = lane & 31, key = KEY_OF_ROW(t >> 4, t & 15);
     lane_at[0] = ((key & 15) * D + (wave * (2 * DC) + (lane >> 5)) * 8) * 2;  // the further chunks: + 32 bytes each
   }
-  const bool second_piece = PF_KEY_OF_ROW((lane & 31) >> 4, lane & 15) >> 4;
+  const bool second_piece = KEY_OF_ROW((lane & 31) >> 4, lane & 15) >> 4;
   auto issue = [&](int step) {
     if ((step & 31) == 0) locate(step >> 5);
     if (wave >= 2) {
@@ -811,7 +814,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       // tile's while they run: a product must not wait for a read issued just before it.
       u32x4_t kraw[2][DC];
       auto read_keys = [&](int tt, u32x4_t (&into)[DC]) {
-        // score tile tt: rows PF_KEY_OF_ROW(tt & 1, .) of step tt >> 1
+        // score tile tt: rows KEY_OF_ROW(tt & 1, .) of step tt >> 1
         const u32x4_t* keys = &lds[(2 * rd + (tt >> 1)) % PF_STAGES][0][0] + (tt & 1) * 16 + col;
 #pragma unroll
         for (int c = 0; c < DC; ++c) into[c] = keys[(c * 4 + grp) * 32];
@@ -842,7 +845,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
           for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int key = kb + 32 * (tt >> 1) + PF_KEY_OF_ROW(tt & 1, 4 * grp + r);
+              const int key = kb + 32 * (tt >> 1) + KEY_OF_ROW(tt & 1, 4 * grp + r);
               const bool seen = key <= qpos[qt] && (window <= 0 || key > qpos[qt] - window);
               sc[qt][tt][r] = seen ? sc[qt][tt][r] : NEG_INF;
             }
