@@ -191,8 +191,17 @@ class DecodeGraphs:
         finally:
             if collecting:
                 gc.enable()
-        self.bytes_held += max(0, torch.cuda.memory_reserved() - before)
+        self.bytes_held = self._bytes_now(self.bytes_held + max(0, torch.cuda.memory_reserved() - before))
         return graph, batch, out
+
+    def _bytes_now(self, otherwise: int) -> int:
+        """The shared logits plus the segments of the captures' memory pool (which nothing else can use
+        while the graphs live); `otherwise` where the allocator does not tell segments by pool."""
+        held = self.logits.numel() * self.logits.element_size()
+        segments = torch.cuda.memory_snapshot()
+        if not segments or "segment_pool_id" not in segments[0]:
+            return otherwise
+        return held + sum(s["total_size"] for s in segments if tuple(s["segment_pool_id"]) == tuple(self.pool))
 
     @torch.inference_mode()
     def capture_ahead(self, max_rows: int) -> int:

@@ -484,6 +484,9 @@ def test_a_step_sent_ahead_may_be_the_first_of_its_graph(tmp_path):
         engine.run_ahead = run_ahead
         outs.append(engine.generate(prompts, params))
         assert len(engine.runner.decode_graphs.graphs) == 2 and engine.stats()["kv_blocks_used"] == 0
+        # what the captured steps hold is reported: at least their logits, also when the allocator had room to spare
+        logits_bytes = engine.runner.decode_graphs.most_rows * raw["vocab_size"] * 4
+        assert engine.stats()["graph_bytes"] >= logits_bytes
     assert outs[0] == outs[1] and all(len(o) == 24 for o in outs[0])
 
 
