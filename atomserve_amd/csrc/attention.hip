@@ -357,12 +357,25 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const int* __restrict__ items, const int* __restrict__ positions, const int* __restrict__ tok_row,
     const int* __restrict__ block_tables, int table_width, bf16* __restrict__ out, float* __restrict__ part_m,
     float* __restrict__ part_l, float* __restrict__ part_acc, int H, int KV, int bs, float scale, int window,
-    int part_size, int P, FreshQKV fresh) {
+    int part_size, int P, int cus, FreshQKV fresh) {
   constexpr int D = DC * 32, DT = DC * 2;  // DT: tiles of 16 output coordinates
   extern __shared__ float smem[];          // [4][16] m, [4][16] l, [4][D][G] acc
   __shared__ __align__(16) bf16 fresh_kv[2][256];  // FRESH: the new token's key and value
   const int G = H / KV;
-  const int item = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;
+  int item = blockIdx.x, kvh = blockIdx.y;
+  const int part = blockIdx.z;
+  if (P == 1) {
+    // Whole contexts, one workgroup each, of unequal length: two workgroups share a compute unit, and
+    // the first two rounds of `cus` workgroups are placed at once, the second on top of the first.
+    // Work is taken in the order (item, kv head) with the second round backwards, so that with
+    // `items` sorted longest first a compute unit's first two are the longest with the shortest of
+    // those 2 cus; what follows goes to whichever compute unit is free, longest first.
+    int s = blockIdx.x + gridDim.x * blockIdx.y;
+    const int total = gridDim.x * gridDim.y;
+    if (s >= cus && s < 2 * cus) s = cus + (min(2 * cus, total) - 1 - s);
+    item = s / KV;
+    kvh = s % KV;
+  }
   const int t = items ? items[item] : item;  // null: every token, in order
   const int pos = positions[t];
   const int ctx = pos + 1;
@@ -968,7 +981,7 @@ static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_
   attn_decode_mfma_kernel<DCV, FRESHV><<<grid, 256, shmem, stream>>>(                                     \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, items, positions, tok_row, block_tables, \
       table_width, (bf16*)out, part_m, part_l, part_acc, H, KV, bs, scale, window, part_size, P,          \
-      FRESHV ? *fresh : none)
+      compute_units(), FRESHV ? *fresh : none)
 #define LAUNCH_FRESH(FRESHV)            \
   switch (D / 64) {                     \
     case 1: LAUNCH(2, FRESHV); break;   \
@@ -1020,10 +1033,11 @@ extern "C" int as_attn_decode_mfma(const void* q, const void* k_pages, const voi
 // A decode step (token t is row t of the block tables) from the projection's output: per-head norm,
 // rotation of the whole head, the new token's key and value written to its slot (store 0: queries
 // only, the pages already hold them), and attention, in one kernel.  qkv [T, H + 2 KV, D] bf16;
-// qw, kw [D] bf16 or fp32; cs [T, D/2] float2; slots [T].  Needs D % 64 == 0.
+// qw, kw [D] bf16 or fp32; cs [T, D/2] float2; slots [T]; items [T]: the order in which the tokens are
+// taken (null: as they come), best the longest contexts first.  Needs D % 64 == 0.
 extern "C" int as_attn_decode_fresh(const void* qkv, const void* qw, const void* kw, int gains_dtype,
                                     const float* cs, const int* slots, float eps, int store, void* k_pages,
-                                    void* v_pages, int num_tokens, const int* positions,
+                                    void* v_pages, const int* items, int num_tokens, const int* positions,
                                     const int* block_tables, int table_width, void* out, float* part_m,
                                     float* part_l, float* part_acc, int H, int KV, int D, int bs, float scale,
                                     int window, int part_size, int P, hipStream_t stream) {
@@ -1035,7 +1049,7 @@ extern "C" int as_attn_decode_fresh(const void* qkv, const void* qw, const void*
   if (gains_dtype != DT_BF16 && gains_dtype != DT_F32) return AS_BAD_DTYPE;
   const FreshQKV fresh = {(const bf16*)qkv, qw, kw, (const float2*)cs, slots, (bf16*)k_pages, (bf16*)v_pages,
                           eps, store};
-  return launch_decode_mfma(nullptr, k_pages, v_pages, nullptr, num_tokens, positions, nullptr, block_tables,
+  return launch_decode_mfma(nullptr, k_pages, v_pages, items, num_tokens, positions, nullptr, block_tables,
                             table_width, out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size,
                             P, &fresh, gains_dtype, stream);
 }

@@ -68,7 +68,8 @@ class StepBatch:
     token_ids, positions, tok_row [T] int32   (tok_row: which row a token belongs to)
     logits_rows [B'] int32                    flat indices of the wanted positions
     group_slots[g] [T], group_tables[g] [R, W_g] int32, per paged group
-    all_tokens [T]; with row_split = (short, tile), as the model's mixers ask (`Mixer.row_split`):
+    all_tokens [T]: every token (in a decode step those with the longest contexts first);
+    with row_split = (short, tile), as the model's mixers ask (`Mixer.row_split`):
     short_tokens [Ns]: tokens of rows with <= short tokens;
     long_tiles [Nt, 4]: (first flat token, count, row, first position) per `tile` queries of longer rows
     row_first, row_len, row_start, row_slots [R] int32 (for mixers with per-request state)
@@ -156,8 +157,13 @@ class StepBatch:
                 arr[r, : len(t)] = [0 if p == RELEASED else p for p in t]
             tables.append(arr)
 
+        # Every token; in a decode step those that see most keys first, the order in which the attention
+        # kernel's workgroups take whole contexts (`advance` keeps it: the contexts grow together).
+        every = range(T)
+        if T == R and T > 1:
+            every = np.argsort(-np.asarray(pos, dtype=np.int64), kind="stable")
         fields = [("token_ids", tok), ("positions", pos), ("tok_row", trow), ("logits_rows", want),
-                  ("all_tokens", range(T)), ("short_tokens", short), ("long_tiles", tiles),
+                  ("all_tokens", every), ("short_tokens", short), ("long_tiles", tiles),
                   ("row_first", row_first), ("row_len", row_len), ("row_start", row_start),
                   ("row_slots", row_slots)]  # fmt: skip
         for g in range(num_paged_groups):

@@ -274,13 +274,15 @@ def attn_decode_fresh_supported(dtype, num_heads: int, num_kv_heads: int, head_d
 
 
 def attn_decode_fresh(qkv, q_weight, k_weight, cos_sin, slots, eps, store_kv, k_pages, v_pages, positions,
-                      block_tables, out, num_heads, scale, window, max_context, part_size=None) -> None:
+                      block_tables, out, num_heads, scale, window, max_context, part_size=None, order=None) -> None:
     """A decode step from the projection's output, in one kernel: what `qk_norm_rope_store` and then
     `attn_single_query` do for tokens that are their own rows (token t reads block table t).
 
     qkv [T, H + 2 KV, D] bf16; q_weight, k_weight [D] bf16 or fp32; cos_sin [T, D/2, 2] fp32;
     slots [T] int32; store_kv False: queries only, the pages already hold the tokens' keys and values
-    (a run that reads another run's cache); out [T, H, D]."""
+    (a run that reads another run's cache); out [T, H, D]; order [T] int32: the tokens in the order in
+    which the workgroups take them (a permutation; longest contexts first keeps the compute units evenly
+    busy when whole contexts are walked), None: as they come."""
     _check(qkv, "qkv", BF16, (None, None, None))
     T, heads, D = qkv.shape
     H = num_heads
@@ -304,13 +306,16 @@ def attn_decode_fresh(qkv, q_weight, k_weight, cos_sin, slots, eps, store_kv, k_
     w_dtype = q_weight.dtype
     if store_kv:
         _check(slots, "slots", I32, (T,))
+    if order is not None:
+        _check(order, "order", I32, (T,))
     if T == 0:
         return
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
     part_size, P, part_m, part_l, part_acc = _partitions(T, H, KV, D, max_context, window, True, part_size, qkv.device)
     call("as_attn_decode_fresh", _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _DT[w_dtype], _ptr(cos_sin),
-         _ptr(slots) if store_kv else 0, float(eps), int(bool(store_kv)), _ptr(k_pages), _ptr(v_pages), T,
+         _ptr(slots) if store_kv else 0, float(eps), int(bool(store_kv)), _ptr(k_pages), _ptr(v_pages),
+         _ptr(order) if order is not None else 0, T,
          _ptr(positions), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
          _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
 PREFILL_TILE_QUERIES = 64  # queries of one work item of the prefill kernel

@@ -84,7 +84,7 @@ class Attention(Mixer):
             ops.attn_decode_fresh(
                 qkv.view(T, H + 2 * KV, D), self.q_norm_weight, self.k_norm_weight, cos_sin, cache.slots, eps,
                 cache.writes, cache.k_pages, cache.v_pages, step.positions, cache.block_tables, out, H, s.scale,
-                s.window, step.max_context,
+                s.window, step.max_context, order=step.all_tokens,
             )  # fmt: skip
         else:
             q = torch.empty((T, H, D), dtype=env.dtype, device=device)
@@ -111,8 +111,8 @@ class Attention(Mixer):
         # fp32, and shapes the prefill kernel does not take: every token is a single query.
         # Otherwise short rows are single queries and long rows go through the prefill kernel.
         if step.decode_only:  # token t is row t: the kernels need no maps from one to the other
-            ops.attn_single_query(q, cache.k_pages, cache.v_pages, None, step.positions, None, cache.block_tables,
-                                  out, s.scale, s.window, step.max_context)  # fmt: skip
+            ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, None,
+                                  cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
             return
         if not ops.attn_prefill_supported(self.env.dtype, s.head_dim, cache.block_size):
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,

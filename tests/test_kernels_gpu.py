@@ -597,6 +597,42 @@ def test_attention_of_a_decode_step_needs_no_maps(ops, dtype):
         ops.attn_single_query(q, k_pages, v_pages, None, positions, None, tables[:3], b, D**-0.5, 0, max(lens))
 
 
+@pytest.mark.parametrize("N,KV", [(40, 8), (100, 8), (70, 3), (300, 2), (5, 8)])
+def test_whole_contexts_in_a_given_order(ops, N, KV):
+    """Single queries over whole contexts (no partitions), more workgroups than one, two and three rounds
+    of one per compute unit, taken in the order of a permutation (longest first, as a decode step packs
+    them, and a random one): every token is attended exactly once, by both kernels' entry points."""
+    H, D, bs = 2 * KV, 64, 16
+    torch.manual_seed(N)
+    lens = torch.randint(1, 200, (N,)).tolist()
+    q, k_pages, v_pages, tables, positions = paged_case(BF16, H, KV, D, bs, lens, seed=N, k_scale=3.0 / math.sqrt(D / 16))
+    rows = i32(list(range(N)))
+    scale = D**-0.5
+    ref = pk.paged_attention(q, k_pages, v_pages, rows, positions, rows, tables, scale, 0)
+    whole = -(-max(lens) // 32) * 32
+    longest_first = torch.argsort(positions, descending=True, stable=True).to(torch.int32)
+    shuffled = torch.randperm(N).to(torch.int32).to(DEV)
+    for order in (None, longest_first, shuffled):
+        out = torch.full((N, H, D), float("nan"), dtype=BF16, device=DEV)
+        ops.attn_single_query(q, k_pages, v_pages, order, positions, None, tables, out, scale, 0, max(lens), whole)
+        assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2)
+    # the kernel fed with fresh projections, queries only (the pages hold the keys already)
+    g = torch.Generator().manual_seed(N + 1)
+    qkv = (torch.randn(N, H + 2 * KV, D, generator=g) * 2).to(BF16).to(DEV)
+    qw, kw = (torch.randn(D, generator=g) + 1).to(BF16).to(DEV), (torch.randn(D, generator=g) + 1).to(BF16).to(DEV)
+    inv = (1.0 / (1e4 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))).to(DEV)
+    cs = torch.empty(N, D // 2, 2, device=DEV)
+    ops.rope_table(positions, inv, cs)
+    outs = []
+    for order in (None, longest_first, shuffled):
+        out = torch.full((N, H, D), float("nan"), dtype=BF16, device=DEV)
+        ops.attn_decode_fresh(qkv, qw, kw, cs, None, 1e-6, False, k_pages, v_pages, positions, tables, out, H, scale, 0,
+                              max(lens), whole, order=order)
+        outs.append(out)
+    assert not torch.isnan(outs[0].float()).any()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
 @pytest.mark.parametrize("H,KV,D,bs,gain,window", [
     (32, 8, 128, 16, BF16, 0), (6, 2, 64, 32, F32, 0), (14, 2, 192, 16, BF16, 40), (5, 5, 256, 16, BF16, 0),
     (16, 1, 128, 48, F32, 0), (8, 2, 128, 16, BF16, 1),
