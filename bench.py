@@ -13,6 +13,7 @@ ignore_eos, warm-up first, prompt steps outside the decode timer, tokens counted
 import argparse
 import json
 import os
+import random
 import sys
 import time
 
@@ -44,6 +45,8 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=8)
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=2048)
+    p.add_argument("--shortest-context", type=int, default=0, help="contexts spread evenly from this many tokens to "
+                   "--context over the batch instead of all equal (0: equal)")
     p.add_argument("--sizes", choices=sorted(SIZES), default="8b", help="layer sizes of Qwen3-8B, -0.6B or -32B")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both counts are reported)")
     p.add_argument("--max-len", type=int, default=4096, help="longest sequence the cache pool is sized for")
@@ -222,13 +225,16 @@ def main() -> int:
 
     def run_decode(batch: int, steps: int, warmup: int, profile: int = 0):
         """Prefill `batch` prompts of args.context tokens (untimed), then time `steps` decode steps."""
-        handles = [engine.submit(prompt(b, args.context, c.vocab_size), params) for b in range(batch)]
+        lo = args.shortest_context or args.context
+        lengths = [lo + (args.context - lo) * b // max(1, batch - 1) for b in range(batch)]
+        random.Random(0).shuffle(lengths)
+        handles = [engine.submit(prompt(b, n, c.vocab_size), params) for b, n in enumerate(lengths)]
         while any(s.num_computed_tokens < s.num_prompt_tokens for s in
                   [*engine.scheduler.running, *engine.scheduler.waiting]) or engine.scheduler.waiting or not engine.scheduler.running:
             engine.step()
         for _ in range(warmup):
             engine.step()
-        ctx_start = engine.scheduler.running[0].num_tokens
+        ctx_start = sum(s.num_tokens for s in engine.scheduler.running) / batch
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
@@ -293,7 +299,7 @@ def main() -> int:
             "model": f"Qwen3-{args.sizes.upper()} sizes", "layers": c.num_layers, "layers_full": full_layers, "hidden": c.hidden_size,
             "heads": c.num_heads, "kv_heads": c.num_kv_heads, "head_dim": c.head_dim,
             "intermediate": c.intermediate_size, "vocab": c.vocab_size, "global_batch": args.batch,
-            "seq_len": args.context, "max_context": max_len, "block_size": block, "parallelism": "single GPU",
+            "seq_len": args.context, "shortest_context": args.shortest_context or args.context, "max_context": max_len, "block_size": block, "parallelism": "single GPU",
             "sampling": "greedy" if args.greedy else "temperature 0.6 top-k 20 top-p 0.95",
         },
         "roofline": roofline(args.batch, mean_ctx, ms),
