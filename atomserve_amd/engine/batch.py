@@ -144,6 +144,7 @@ class StepBatch:
         # Work items of the prefill kernel, the ones that see most keys first: the kernel hands
         # them out in this order and pairs the longest with the shortest on a compute unit.
         tile_list.sort(key=lambda t: -(t[3] + t[1]))
+        short.sort(key=lambda t: -pos[t])  # single queries too: the longest contexts first
         tiles = [v for t in tile_list for v in t]
         self.max_context = max(self.max_context, max_context)
         self.max_short_context = max(self.max_short_context, max_context if short else 0)

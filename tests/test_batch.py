@@ -27,7 +27,7 @@ def test_rows_are_flattened_with_slots_tables_and_tiles():
     assert b.group_slots[0].tolist() == [2 * BS + 0, 2 * BS + 1, 2 * BS + 2, 3 * BS + 2]
     assert b.group_slots[1].tolist() == [1 * BS + 0, 1 * BS + 1, 1 * BS + 2, 4 * BS + 2]
     assert b.group_tables[0].tolist() == [[5, 2], [3, 0]]
-    assert b.short_tokens.tolist() == [0, 1, 2, 3] and b.num_long_tiles == 0
+    assert b.short_tokens.tolist() == [2, 1, 0, 3] and b.num_long_tiles == 0  # those that see most keys first
     long = pack([Row(list(range(70)), 0, [list(range(20)), list(range(20))], []), Row([1] * 9, 64, [list(range(20, 40))] * 2, [])])
     # work items of the prefill kernel, the one that sees most keys first
     assert long.long_tiles.tolist() == [[70, 9, 1, 64], [64, 6, 0, 64], [0, 64, 0, 0]]
@@ -74,6 +74,17 @@ def test_a_repeated_decode_step_is_updated_in_place():
     tables[0][0][2] = 6
     assert batch.advance(decode_rows(tables, [8, 5], [1, 2], filler))
     assert not batch.advance(decode_rows(tables, [12, 6], [1, 2], filler))  # beyond the packed table width
+
+
+def test_a_decode_step_lists_its_tokens_longest_context_first():
+    """`all_tokens` of a step of single tokens is the order in which the attention kernel takes whole contexts:
+    most keys first, equal ones as they come; a step with a prompt lists its tokens as they are."""
+    filler = [[0], [0]]
+    tables = [[[5, 2, 6], [7, 1, 3]]] * 4
+    batch = pack(decode_rows(tables, [2, 9, 5, 9], [1, 2, 3, 4], filler), table_width=3, max_context=12)
+    assert batch.decode_only and batch.all_tokens.tolist() == [1, 3, 2, 0, 4]
+    mixed = pack([Row([1, 2, 3], 0, tables[0], [2]), Row([4], 9, tables[1], [0])])
+    assert not mixed.decode_only and mixed.all_tokens.tolist() == [0, 1, 2, 3]
 
 
 def test_rows_are_sorted_only_for_mixers_that_ask():
