@@ -367,14 +367,16 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   if (P == 1) {
     // Whole contexts, one workgroup each, of unequal length: two workgroups share a compute unit, and
     // the first two rounds of `cus` workgroups are placed at once, the second on top of the first.
-    // Work is taken in the order (item, kv head) with the second round backwards, so that with
-    // `items` sorted longest first a compute unit's first two are the longest with the shortest of
-    // those 2 cus; what follows goes to whichever compute unit is free, longest first.
+    // Work is taken eight items at a time, their kv heads one after the other (so neighbours in this
+    // order read different pages at the same time), with the second round backwards: with `items`
+    // sorted longest first a compute unit's first two are a long and a short one, and what follows
+    // goes to whichever compute unit is free, longest first.
     int s = blockIdx.x + gridDim.x * blockIdx.y;
     const int total = gridDim.x * gridDim.y;
     if (s >= cus && s < 2 * cus) s = cus + (min(2 * cus, total) - 1 - s);
-    item = s / KV;
-    kvh = s % KV;
+    const int N = gridDim.x, first = s / (8 * KV) * 8, r = s % (8 * KV), here = min(8, N - first);
+    item = first + r % here;
+    kvh = r / here;
   }
   const int t = items ? items[item] : item;  // null: every token, in order
   const int pos = positions[t];

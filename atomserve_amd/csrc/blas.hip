@@ -11,6 +11,7 @@
 #include "common.h"
 
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <map>
 #include <mutex>
@@ -74,6 +75,39 @@ extern "C" int as_blas_plan(int M, int N, int K, int out_dtype, size_t workspace
   if (M <= 0 || N <= 0 || K <= 0 || (out_dtype != DT_BF16 && out_dtype != DT_F32)) return 0;
   Plan* plan = plan_for(M, N, K, out_dtype, workspace_bytes);
   return plan ? (int)plan->candidates.size() : 0;
+}
+
+// The library's own number of a candidate's kernel (the same number names the same kernel for every
+// shape, within one version of the library), -1 if there is none.
+extern "C" int as_blas_candidate_index(int M, int N, int K, int out_dtype, size_t workspace_bytes, int candidate) {
+  Plan* plan = plan_for(M, N, K, out_dtype, workspace_bytes);
+  if (!plan || candidate < 0 || candidate >= (int)plan->candidates.size()) return -1;
+  return hipblaslt_ext::getIndexFromAlgo(plan->candidates[candidate].algo);
+}
+
+// Makes the kernel with the library's number `index` (as_blas_candidate_index of another shape's
+// candidate) a candidate of this shape: returns its place among the shape's candidates, adding it
+// if the library says it can compute this shape within the workspace, or -1 if it cannot.
+extern "C" int as_blas_adopt(int M, int N, int K, int out_dtype, size_t workspace_bytes, int index) {
+  Plan* plan = plan_for(M, N, K, out_dtype, workspace_bytes);
+  if (!plan || index < 0) return -1;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (size_t i = 0; i < plan->candidates.size(); ++i)
+    if (hipblaslt_ext::getIndexFromAlgo(plan->candidates[i].algo) == index) return (int)i;
+  std::vector<int> wanted = {index};
+  std::vector<hipblasLtMatmulHeuristicResult_t> found;
+  if (!ok(hipblaslt_ext::getAlgosFromIndex(g_handle, wanted, found))) return -1;
+  const float one = 1.f, zero = 0.f;
+  for (auto& result : found) {
+    size_t needs = 0;
+    if (ok(hipblaslt_ext::matmulIsAlgoSupported(g_handle, plan->desc, &one, plan->a, plan->b, &zero, plan->c, plan->c,
+                                                result.algo, needs)) &&
+        needs <= workspace_bytes) {
+      plan->candidates.push_back(result);
+      return (int)plan->candidates.size() - 1;
+    }
+  }
+  return -1;
 }
 
 // Runs candidate `candidate` of the shape's plan.  a [M, K], w [N, K] bf16; out [M, N] bf16 or fp32;

@@ -293,6 +293,30 @@ class ModelRunner:
         graphs = self.decode_graphs
         return graphs is not None and graphs.eligible([graphs.filler()] * len(seqs))
 
+    @torch.inference_mode()
+    def tune_prompt_lengths(self, most_tokens: int) -> list:
+        """Runs a prompt that stores nothing at each of a few lengths (128, 192, 256, 384, ... up to `most_tokens`)
+        until the library's candidates for its products have been tried and the fastest chosen; prompts
+        of other lengths then take what the next length above them chose.  Returns the lengths run."""
+        if self.device.type != "cuda" or ops.library_choices_fixed():
+            return []
+        bs, lengths, n = self.manager.block_size, [], 128
+        while n <= most_tokens:
+            lengths.extend(m for m in (n, n + n // 2) if m <= most_tokens)
+            n *= 2
+        slot = self.pools.scrap_slot if self.manager.state_groups else -1
+        for n in lengths:
+            ops.tune_library_rows(n)
+            tables = [[0] * -(-n // bs) for _ in self.manager.paged_groups]
+            rows = [Row([0] * n, 0, tables, [n - 1], slot, store=False)]
+            for _ in range(4):
+                self.step(rows)
+                if not ops.library_trials_pending():
+                    break
+            ops.settle_library_choices()
+        torch.cuda.synchronize()
+        return lengths
+
     def graph_bytes(self) -> int:
         """Device memory that captured decode steps hold (their shared logits and memory pool)."""
         return 0 if self.decode_graphs is None else self.decode_graphs.bytes_held

@@ -406,9 +406,14 @@ def gemm(a, w, out) -> None:
 # not its fastest on this GPU, so the first calls of such a shape try the candidates in turn, each
 # on the weights of the layer that happens to call (cold, as every decode step meets them), timed
 # by events in place; when every candidate has run LIBRARY_TRIALS_EACH times (the first run of a
-# kernel is slow), or a capture begins, the fastest stays.
+# kernel is slow), or a capture begins, the fastest stays.  The same is done for the row counts that
+# `tune_library_rows` names (the token budget of a step; lengths of prompts that a warm-up runs), and
+# a product of any other row count above 64 takes the kernel that the nearest tuned row count above
+# it settled on: at 128 rows of Qwen3-8B sizes the library's first candidates take 168 us a layer,
+# the fastest of the first sixteen 132 us.
 LIBRARY_WORKSPACE_BYTES = 64 << 20
 LIBRARY_TUNED_ROWS = {32, 64}
+LIBRARY_DECODE_ROWS = 64  # row counts up to here are decode steps' (padded to 32 and 64)
 LIBRARY_TRIALS_EACH = 4
 _library = {"workspace": None, "choice": {}, "trials": {}, "fixed": False}
 
@@ -420,6 +425,10 @@ def fix_library_choices(fixed: bool = True) -> None:
     _library["fixed"] = bool(fixed)
     if fixed:
         _library["trials"].clear()
+
+
+def library_choices_fixed() -> bool:
+    return _library["fixed"]
 
 
 def library_choices() -> dict:
@@ -450,8 +459,14 @@ def _library_gemm(a, w, out, M, N, K) -> None:
             count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
             if count == 0:
                 choice = state["choice"][key] = -1  # the library offers nothing for this shape through this door
-            elif count == 1 or M not in LIBRARY_TUNED_ROWS or state["fixed"]:
+            elif count == 1 or state["fixed"]:
                 choice = state["choice"][key] = 0  # the library's first candidate, which is what torch.mm runs
+            elif M not in LIBRARY_TUNED_ROWS:
+                choice = _choice_of_tuned_rows(M, N, K, out.dtype)  # a prompt of any length: what its bucket settled on
+                if choice is None:
+                    choice = 0  # nothing settled yet: the first candidate for now, asked again at the next call
+                else:
+                    state["choice"][key] = choice
             else:
                 trial = state["trials"][key] = {"count": count, "runs": []}
         if trial is not None:
@@ -463,6 +478,24 @@ def _library_gemm(a, w, out, M, N, K) -> None:
     if choice < 0:
         return _torch_gemm(a, w, out)
     _library_call(a, w, out, M, N, K, choice)
+
+
+def _choice_of_tuned_rows(M, N, K, dtype):
+    """For a product of a row count that is not tuned itself: the kernel that the nearest tuned row
+    count above it (of more than 64 rows: a prompt's, not a decode step's) settled on for the same
+    weights, as a candidate of this shape; None while that one has not settled, or there is none."""
+    above = [rows for rows in LIBRARY_TUNED_ROWS if rows >= M and rows > LIBRARY_DECODE_ROWS]
+    if not above:
+        return None
+    tuned = min(above)
+    settled = _library["choice"].get((tuned, N, K, dtype))
+    if settled is None:
+        return None
+    if settled < 0:
+        return 0
+    index = entry("as_blas_candidate_index")(tuned, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, settled)
+    place = entry("as_blas_adopt")(M, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, index)
+    return place if place >= 0 else 0
 
 
 def _library_call(a, w, out, M, N, K, candidate) -> None:

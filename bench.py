@@ -93,6 +93,7 @@ def mixed_workload(args, model, config, full_layers: int) -> dict:
     engine = create_engine(model, EngineConfig(block_size=block, num_blocks=requests * max_len // block,
                                                max_num_seqs=requests, max_num_batched_tokens=budget,
                                                max_model_len=max_len, enable_prefix_caching=True), seed=0)  # fmt: skip
+    engine.warm_up()  # as the command line does before it serves
     params = SamplingParams(temperature=0.0, max_tokens=decoded, ignore_eos=True) if args.greedy else \
         SamplingParams(max_tokens=decoded, ignore_eos=True)  # fmt: skip
     rng = random.Random(0)
@@ -206,6 +207,7 @@ def main() -> int:
                                  max_num_batched_tokens=max(2048, args.context), max_model_len=max_len,
                                  enable_prefix_caching=False)  # fmt: skip
     engine = create_engine(model, engine_config, seed=0)
+    engine.warm_up()  # as the command line does before it serves: decode steps captured, prompt lengths tried
 
     itemsize = 2 if args.dtype == "bf16" else 4
     c = config

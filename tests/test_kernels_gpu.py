@@ -372,6 +372,53 @@ def test_every_candidate_of_the_library_gives_the_product(ops):
     assert not ops.library_trials_pending()
 
 
+def test_a_product_of_any_row_count_takes_what_the_tuned_count_above_it_chose(ops):
+    """Prompts come in every length: a product whose row count is not tuned itself runs the kernel that
+    the nearest tuned row count above it settled on (by the library's own number of that kernel), and
+    gives the product; while that one is undecided, and with fixed choices, the first candidate."""
+    from atomserve_amd.kernels.lib import entry
+
+    torch.manual_seed(31)
+    N, K, tuned, M = 1024, 2048, 192, 100
+    w = torch.randn(N, K, device=DEV).to(BF16)
+    a = torch.randn(M, K, device=DEV).to(BF16)
+    out = torch.empty(M, N, dtype=BF16, device=DEV)
+    number = lambda rows, place: entry("as_blas_candidate_index")(rows, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, place)
+    was_fixed = ops.library_choices_fixed()
+    ops.fix_library_choices(False)
+    ops.tune_library_rows(tuned)
+    try:
+        ops.gemm(a, w, out)  # nothing settled above 100 rows: the first candidate, and no decision
+        assert close_bf16(out, pk.gemm(a, w), scale=math.sqrt(K)) and (M, N, K, BF16) not in ops.library_choices()
+        big = torch.randn(tuned, K, device=DEV).to(BF16)
+        big_out = torch.empty(tuned, N, dtype=BF16, device=DEV)
+        while (tuned, N, K, BF16) not in ops.library_choices():
+            ops.gemm(big, w, big_out)
+        chosen = ops.library_choices()[(tuned, N, K, BF16)]
+        out.fill_(float("nan"))
+        ops.gemm(a, w, out)
+        assert close_bf16(out, pk.gemm(a, w), scale=math.sqrt(K))
+        mine = ops.library_choices()[(M, N, K, BF16)]
+        assert number(M, mine) == number(tuned, chosen) or (mine == 0 and entry("as_blas_adopt")(M, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, chosen)) < 0)
+        # a kernel that this shape's own list does not hold is added to it, once
+        count = entry("as_blas_plan")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)
+        for place in range(entry("as_blas_plan")(tuned, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)):
+            at = entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, place))
+            assert at < 0 or number(M + 1, at) == number(tuned, place)
+            assert at == entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, place))
+        grown = entry("as_blas_plan")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)
+        assert grown >= count
+        a1 = torch.randn(M + 1, K, device=DEV).to(BF16)
+        for place in range(count, grown):  # the adopted ones give the product too
+            o1 = torch.zeros(M + 1, N, dtype=BF16, device=DEV)
+            ops._library_call(a1, w, o1, M + 1, N, K, place)
+            assert close_bf16(o1, pk.gemm(a1, w), scale=math.sqrt(K)), place
+        assert entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, -1) < 0
+    finally:
+        ops.LIBRARY_TUNED_ROWS.discard(tuned)
+        ops.fix_library_choices(was_fixed)
+
+
 def test_library_candidates_replay_from_a_graph(ops):
     """Each candidate captured once and replayed with other inputs and a workspace full of noise,
     with eager work and synchronisations between the replays: every replay gives what the eager
