@@ -342,60 +342,60 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_bf16x8_kernel(
   const int hs = (int)(unit % heads);
   const bf16* src = qkv + (t * (H + 2 * KV) + hs) * D;
   const bool is_q = hs < H, is_k = !is_q && hs < H + KV;
+  bf16* dst;
+  if (!is_q && !is_k) {  // values: transposed within the page
+    const int slot = slots[t];
+    if (slot < 0) return;  // uniform over the group
+    const size_t head = (size_t)(slot / block_size) * KV + (hs - H - KV);
+    // A prompt's tokens fill a page slot after slot.  Where eight tokens in a row go to eight
+    // slots in a row that start at a multiple of eight, a coordinate's eight values are 16
+    // contiguous bytes of the transposed page, where token by token they would be eight stores
+    // of two bytes, 2 * block_size bytes apart.  The eight tokens' lane groups share that work:
+    // each takes an eighth of the coordinates, two per lane, reads them from all eight tokens'
+    // rows and stores two 16-byte pieces.
+    const int nth = slot & 7;
+    const long lead = (long)t - nth;
+    bool run = (block_size & 7) == 0 && lead >= 0 && lead + 8 <= (long)(units / heads);
+    if (run) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) run = run && slots[lead + i] == slot - nth + i;
+    }
+    if (run) {  // uniform over the lanes of this (token, head), and the same for all eight tokens
+      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+      const int d0 = nth * (D >> 3) + 2 * l;
+      const bf16* first = qkv + ((size_t)lead * (H + 2 * KV) + hs) * D + d0;
+      bf16x2 pair[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pair[i] = *reinterpret_cast<const bf16x2*>(first + (size_t)i * (H + 2 * KV) * D);
+      bf16x8 oa, ob;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        oa[i] = finite_or_zero((bf16)pair[i][0]);
+        ob[i] = finite_or_zero((bf16)pair[i][1]);
+      }
+      bf16* vt = v_pages + head * block_size * D + (slot - nth) % block_size;
+      *reinterpret_cast<bf16x8*>(vt + (size_t)d0 * block_size) = oa;
+      *reinterpret_cast<bf16x8*>(vt + (size_t)(d0 + 1) * block_size) = ob;
+      return;
+    }
+    const bf16x8 a8 = *reinterpret_cast<const bf16x8*>(src + 8 * l);
+    const bf16x8 b8 = *reinterpret_cast<const bf16x8*>(src + half + 8 * l);
+    bf16* vt = v_pages + head * block_size * D + slot % block_size;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      vt[(size_t)(8 * l + j) * block_size] = finite_or_zero((bf16)a8[j]);
+      vt[(size_t)(half + 8 * l + j) * block_size] = finite_or_zero((bf16)b8[j]);
+    }
+    return;
+  }
   const bf16x8 a8 = *reinterpret_cast<const bf16x8*>(src + 8 * l);
   const bf16x8 b8 = *reinterpret_cast<const bf16x8*>(src + half + 8 * l);
-  bf16* dst;
   if (is_q) {
     dst = q_out + (t * H + hs) * D;
   } else {
     const int slot = slots[t];
     if (slot < 0) return;  // uniform over the group
-    const int kvh = is_k ? hs - H : hs - H - KV;
-    const size_t head = (size_t)(slot / block_size) * KV + kvh;
-    if (!is_k) {  // values: transposed within the page
-      bf16* vt = v_pages + head * block_size * D + slot % block_size;
-      // A prompt's tokens fill a page slot after slot.  Where eight tokens in a row go to eight
-      // slots in a row that start at a multiple of eight, the first of them stores for all:
-      // a coordinate's eight values are 16 contiguous bytes of the transposed page, where token
-      // by token they would be eight stores of two bytes, 2 * block_size bytes apart.
-      const long lead = (long)t - (slot & 7);
-      bool run = (block_size & 7) == 0 && lead >= 0 && lead + 8 <= (long)(units / heads);
-      if (run) {
-        const int first = slot - (slot & 7);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) run = run && slots[lead + i] == first + i;
-      }
-      if (run) {  // uniform over the lanes of this (token, head)
-        if (slot & 7) return;  // the first token of the eight does it
-        bf16x8 va[8], vb[8];
-        va[0] = a8;
-        vb[0] = b8;
-#pragma unroll
-        for (int i = 1; i < 8; ++i) {
-          const bf16* si = src + (size_t)i * (H + 2 * KV) * D;
-          va[i] = *reinterpret_cast<const bf16x8*>(si + 8 * l);
-          vb[i] = *reinterpret_cast<const bf16x8*>(si + half + 8 * l);
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          bf16x8 oa, ob;
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            oa[i] = finite_or_zero((bf16)va[i][j]);
-            ob[i] = finite_or_zero((bf16)vb[i][j]);
-          }
-          *reinterpret_cast<bf16x8*>(vt + (size_t)(8 * l + j) * block_size) = oa;
-          *reinterpret_cast<bf16x8*>(vt + (size_t)(half + 8 * l + j) * block_size) = ob;
-        }
-        return;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        vt[(size_t)(8 * l + j) * block_size] = finite_or_zero((bf16)a8[j]);
-        vt[(size_t)(half + 8 * l + j) * block_size] = finite_or_zero((bf16)b8[j]);
-      }
-      return;
-    }
+    const size_t head = (size_t)(slot / block_size) * KV + (hs - H);
     dst = k_pages + (head * block_size + slot % block_size) * D;
   }
   const W* w = is_q ? qw : kw;
