@@ -807,18 +807,48 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
         __builtin_amdgcn_global_load_lds((global_ptr_t)(src + i * 32), (lds_ptr_t)(dst + i * 64), 16, 0, 0);
     }
   };
+  // The same copies one instruction at a time, for a round's two steps: `aim` works out where they read
+  // and write, `copy(k)` issues the k-th of their 2 DC instructions (between the round's matrix products,
+  // whose issue otherwise leaves the wave idle, instead of in one block that the wave waits through).
+  const char* from[2];
+  u32x4_t* to[2];
+  auto aim = [&](int step0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int step = step0 + j;
+      if ((step & 31) == 0) locate(step >> 5);
+      if (wave >= 2) {
+        from[j] = reinterpret_cast<const char*>(v_pages) + at(v_at, 2 * step + wave - 2);
+        to[j] = &lds[step % PF_STAGES][wave][0];
+      } else {
+        const unsigned long long first = at(k_at, 2 * step), second = at(k_at, 2 * step + 1);
+        from[j] = reinterpret_cast<const char*>(k_pages) + (second_piece ? second : first) + lane_at[0];
+        to[j] = &lds[step % PF_STAGES][0][0] + wave * (DC * 64);
+      }
+    }
+  };
+  auto copy = [&](int k) {
+    const int j = k / DC, i = k % DC;
+    if (wave >= 2) __builtin_amdgcn_global_load_lds((global_ptr_t)(from[j] + lane_at[i]), (lds_ptr_t)(to[j] + i * 64), 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((global_ptr_t)(from[j] + i * 32), (lds_ptr_t)(to[j] + i * 64), 16, 0, 0);
+  };
   const int nrounds = (nsteps + 1) / 2;
   issue(0);
   issue(1);  // beyond the last key it repeats the last piece
   for (int rd = 0; rd < nrounds; ++rd) {
     PF_WAIT_VM(0);    // this wave's copies for the round have landed
     __syncthreads();  // ... and everyone's; and everyone is done with the round before
-    if (rd + 1 < nrounds) {  // into the two stages the round before used
-      issue(2 * rd + 2);
-      issue(2 * rd + 3);
-    }
+    const bool more = rd + 1 < nrounds;  // copies into the two stages the round before used
     const int kb = kb0 + 64 * rd;
-    if (working && kb <= my_last && kb + 63 >= my_lo) {
+    const bool active = working && kb <= my_last && kb + 63 >= my_lo;
+    if (more) {
+      aim(2 * rd + 2);
+      if (!active) {
+#pragma unroll
+        for (int k = 0; k < 2 * DC; ++k) copy(k);
+      }
+    }
+    if (active) {
       // raw scores of 64 keys x 32 queries; a key operand is read from LDS once for both query tiles
       f32x4_t sc[2][4];
 #pragma unroll
@@ -846,6 +876,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
           for (int qt = 0; qt < 2; ++qt)
             sc[qt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[qt][c], sc[qt][tt], 0, 0, 0);
         }
+        if (more) {  // a quarter of the round's copies behind each tile's products
+#pragma unroll
+          for (int k = tt * (2 * DC) / 4; k < (tt + 1) * (2 * DC) / 4; ++k) copy(k);
+        }
       }
       // Only rounds that touch the causal diagonal, the window's edge or the end of the context
       // need a mask; the others see all 64 keys (uniform over the wave).
@@ -872,23 +906,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
         const float mx = quad_rows_max(max3(max3(m0, m1, m2), max3(m3, m4, sc[qt][3][3]), NEG_INF));
         // base-2 softmax: scale and log2(e) are folded into one factor (positive, so maxima agree)
         const float mn = fmaxf(m[qt], mx * scale2);
-        float rs = 0.f;
-        alpha[qt] = 1.f;
-        if (mn == NEG_INF) {
+        // Without a branch, so that the two query tiles' arithmetic can be interleaved: while a row
+        // has seen no key, every score and mn are -inf, and 2^(-inf - 0) = 0 is what each weight and
+        // the factor of the (empty) past should be.
+        const float base = mn == NEG_INF ? 0.f : mn;
+        alpha[qt] = __builtin_amdgcn_exp2f(m[qt] - base);
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pop[qt][0][j] = pop[qt][1][j] = (bf16)0.f;
-        } else {
-          alpha[qt] = __builtin_amdgcn_exp2f(m[qt] - mn);  // 2^-inf = 0 while nothing was seen
+        for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-          for (int tt = 0; tt < 4; ++tt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float pv = __builtin_amdgcn_exp2f(fmaf(sc[qt][tt][r], scale2, -mn));
-              rs += pv;
-              pop[qt][tt >> 1][(tt & 1) * 4 + r] = (bf16)pv;
-            }
-          m[qt] = mn;
-        }
+          for (int r = 0; r < 4; ++r) {
+            const float pv = __builtin_amdgcn_exp2f(fmaf(sc[qt][tt][r], scale2, -base));
+            part[r] += pv;
+            pop[qt][tt >> 1][(tt & 1) * 4 + r] = (bf16)pv;
+          }
+        const float rs = (part[0] + part[1]) + (part[2] + part[3]);
+        m[qt] = mn;
         l[qt] = l[qt] * alpha[qt] + quad_rows_sum(rs);
         rescale = rescale || alpha[qt] != 1.f;
       }
