@@ -90,7 +90,7 @@ class DecodeGraphs:
     them); at most `MAX_GRAPHS` are kept, the one replayed longest ago goes first.  `bytes_held`
     is the memory the captures took from the device."""
 
-    ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+    ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256)
     CONTEXT_STEP = 1024
     MAX_GRAPHS = 64
 

@@ -412,8 +412,8 @@ def gemm(a, w, out) -> None:
 # it settled on: at 128 rows of Qwen3-8B sizes the library's first candidates take 168 us a layer,
 # the fastest of the first sixteen 132 us.
 LIBRARY_WORKSPACE_BYTES = 64 << 20
-LIBRARY_TUNED_ROWS = {32, 64}
-LIBRARY_DECODE_ROWS = 64  # row counts up to here are decode steps' (padded to 32 and 64)
+LIBRARY_TUNED_ROWS = {32, 48, 64}
+LIBRARY_DECODE_ROWS = 64  # row counts up to here are decode steps' (padded to 32, 48 and 64)
 LIBRARY_TRIALS_EACH = 4
 _library = {"workspace": None, "choice": {}, "trials": {}, "fixed": False}
 
