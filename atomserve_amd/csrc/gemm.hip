@@ -511,7 +511,7 @@ extern "C" int as_gemm_bf16_scaled(const void* scaled, const float* ssq, int str
                : dispatch_pipe<false, bf16, true, false>(scaled, w, out, M, N, K, stream, link);
 }
 
-// ---- bf16, 17 to 64 rows: tiles of weight rows with the activations staged in LDS ----------
+// ---- bf16, 17 to 128 rows: tiles of weight rows with the activations staged in LDS ---------
 //
 // With more than 16 rows the activations no longer fit a wave's registers, and reading them from
 // memory again for every strip of 16 weight rows costs as much as reading weights (a 16-byte load
@@ -725,7 +725,8 @@ static int launch_tile(const void* a, const void* w, void* out, float* partial, 
   return launch_status();
 }
 
-// out[M, N] = a[M, K] @ w[N, K]^T for 1 <= M <= 64 and K % 256 == 0 through the tile kernel.
+// out[M, N] = a[M, K] @ w[N, K]^T for 1 <= M <= 128 and K % 256 == 0 through the tile kernel
+// (row tiles of 16 up to 64 rows, 96 or 128 rows above; two chunks of 128 rows take 128 KB of LDS).
 //   gated != 0:  w is [2 N, K] (gate rows, then up rows), out[M, N] = silu(gate) * up, bf16.
 //   splits > 0:  K is cut into `splits` ranges (each a multiple of 256) and the fp32 sums of every
 //                range go to partial[splits, M, N]; `out` is not written.
@@ -733,19 +734,22 @@ static int launch_tile(const void* a, const void* w, void* out, float* partial, 
 extern "C" int as_gemm_bf16_tile(const void* a, const void* w, void* out, float* partial, int out_dtype, int M,
                                  int N, int K, int gated, int splits, int strips, hipStream_t stream) {
   if (M <= 0) return AS_OK;
-  if (M > 64 || N <= 0 || K <= 0 || (K % TILE_KC) || splits < 0) return AS_BAD_SHAPE;
+  if (M > 128 || N <= 0 || K <= 0 || (K % TILE_KC) || splits < 0) return AS_BAD_SHAPE;
   if (splits > 0 && (gated || !partial || (K % (splits * TILE_KC)))) return AS_BAD_SHAPE;
   if (splits == 0 && !out) return AS_BAD_SHAPE;
   if (strips == 0) strips = 8;
   if (strips != 8 && strips != 6 && strips != 4 && strips != 2) return AS_BAD_SHAPE;
   if ((unsigned long long)(gated ? 2 : 1) * N * K * 2ull > 0xf0000000ull) return AS_BAD_SHAPE;  // 32-bit byte offsets
-  const int MT = (M + 15) / 16;
+  int MT = (M + 15) / 16;
+  if (MT > 4) MT = MT <= 6 ? 6 : 8;  // above 64 rows: tiles of 96 and 128 rows
 #define TILE_CASE(MTV, NSV) \
   if (MT == MTV && strips == NSV) return launch_tile<MTV, NSV>(a, w, out, partial, out_dtype, M, N, K, gated, splits, stream)
   TILE_CASE(1, 8); TILE_CASE(2, 8); TILE_CASE(3, 8); TILE_CASE(4, 8);
   TILE_CASE(1, 6); TILE_CASE(2, 6); TILE_CASE(3, 6); TILE_CASE(4, 6);
   TILE_CASE(1, 4); TILE_CASE(2, 4); TILE_CASE(3, 4); TILE_CASE(4, 4);
   TILE_CASE(1, 2); TILE_CASE(2, 2); TILE_CASE(3, 2); TILE_CASE(4, 2);
+  TILE_CASE(6, 8); TILE_CASE(8, 8); TILE_CASE(6, 6); TILE_CASE(8, 6);
+  TILE_CASE(6, 4); TILE_CASE(8, 4); TILE_CASE(6, 2); TILE_CASE(8, 2);
 #undef TILE_CASE
   return AS_BAD_SHAPE;
 }

@@ -164,6 +164,7 @@ class DecodeGraphs:
             self.logits = torch.empty((self.most_rows, r.vocab_size), dtype=torch.float32, device=r.device)
         batch = r.prepare([self.filler() for _ in range(n)], table_width=width, max_context=context)
         out = self.logits[:n]
+        ops.tune_library_rows(n)  # a bucket's products come again at every replay: worth trying the library's candidates
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):

@@ -401,16 +401,16 @@ def gemm(a, w, out) -> None:
 # ---- the library's product, called directly -------------------------------------------------
 #
 # hipBLASLt through `csrc/blas.hip` instead of torch.mm: the same kernels for two thirds of the
-# time on the host.  For the row counts of LIBRARY_TUNED_ROWS (decode steps of 17 to 64 requests
-# are padded to these and replayed thousands of times) the library's first candidate is often
-# not its fastest on this GPU, so the first calls of such a shape try the candidates in turn, each
-# on the weights of the layer that happens to call (cold, as every decode step meets them), timed
-# by events in place; when every candidate has run LIBRARY_TRIALS_EACH times (the first run of a
-# kernel is slow), or a capture begins, the fastest stays.  The same is done for the row counts that
-# `tune_library_rows` names (the token budget of a step; lengths of prompts that a warm-up runs), and
-# a product of any other row count above 64 takes the kernel that the nearest tuned row count above
-# it settled on: at 128 rows of Qwen3-8B sizes the library's first candidates take 168 us a layer,
-# the fastest of the first sixteen 132 us.
+# time on the host.  For the row counts of LIBRARY_TUNED_ROWS (decode steps of 17 and more requests
+# are padded to a few row counts, which the capture of such a step adds here, and replayed thousands
+# of times) the library's first candidate is often not its fastest on this GPU, so the first calls
+# of such a shape try the candidates in turn, each on the weights of the layer that happens to call
+# (cold, as every decode step meets them), timed by events in place; when every candidate has run
+# LIBRARY_TRIALS_EACH times (the first run of a kernel is slow), or a capture begins, the fastest
+# stays.  The same is done for the row counts that `tune_library_rows` names (the token budget of a
+# step; lengths of prompts that a warm-up runs), and a product of any other row count above 64 takes
+# the kernel that the nearest tuned row count above it settled on: at 128 rows of Qwen3-8B sizes the
+# library's first candidates take 168 us a layer, the fastest of the first sixteen 132 us.
 LIBRARY_WORKSPACE_BYTES = 64 << 20
 LIBRARY_TUNED_ROWS = {32, 48, 64}
 LIBRARY_DECODE_ROWS = 64  # row counts up to here are decode steps' (padded to 32, 48 and 64)
@@ -565,12 +565,17 @@ def _fastest_of(trial) -> int:
 
 
 # ---- 17 to 64 rows: tiles of weight rows with the activations staged in LDS ---------------------
+# (the product cut along K, whose partial sums the next norm adds up, up to 128 rows: there the
+# library needs 42 us for Qwen3-8B's down projection and 21 for o, this kernel 24 on average; the
+# gated product of 96 and 128 rows is the library's with the activation after it, 48 and 56 us
+# against 51 and 61)
 TILE_MAX_ROWS = 64
+TILE_SPLIT_MAX_ROWS = 128
 TILE_CHUNK = 256  # K comes in chunks of this many
 
 
-def _tile_rows(rows: int, k: int, dtype) -> bool:
-    return dtype == BF16 and SKINNY_MAX_ROWS < rows <= TILE_MAX_ROWS and k % TILE_CHUNK == 0
+def _tile_rows(rows: int, k: int, dtype, most: int = TILE_MAX_ROWS) -> bool:
+    return dtype == BF16 and SKINNY_MAX_ROWS < rows <= most and k % TILE_CHUNK == 0
 
 
 def _gated_tile_strips(rows: int, outputs: int) -> int:
@@ -588,7 +593,7 @@ def gemm_split_plan(rows: int, n: int, k: int, dtype):
     """(strips, splits) of `gemm_split` for a product of these sizes, or None where it has no kernel:
     tiles of 64 weight rows, and K cut into as many ranges (of whole chunks) as fill the compute
     units with those tiles."""
-    if not _tile_rows(rows, k, dtype) or n % 4:
+    if not _tile_rows(rows, k, dtype, TILE_SPLIT_MAX_ROWS) or n % 4:
         return None
     strips = 4
     tiles = -(-n // (16 * strips))
@@ -600,7 +605,7 @@ def gemm_split_plan(rows: int, n: int, k: int, dtype):
 
 def gemm_split(a, w, plan=None):
     """The fp32 partial sums [splits, M, N] of a[M, K] @ w[N, K]^T with K cut into `splits` ranges;
-    whoever takes them adds them up (`rmsnorm(..., split_sums=)`).  bf16, 17 to 64 rows."""
+    whoever takes them adds them up (`rmsnorm(..., split_sums=)`).  bf16, 17 to 128 rows."""
     _check(a, "a", BF16, (None, None))
     M, K = a.shape
     _check(w, "w", BF16, (None, K))

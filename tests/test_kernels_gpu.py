@@ -949,8 +949,9 @@ def test_sampling_is_seeded_per_request_and_mixes_greedy_rows(ops):
     assert alone == crowd and len(set(alone)) > 1
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 96, 256), (33, 1000, 512), (64, 4096, 1024), (48, 520, 768), (20, 64, 3072), (64, 12, 256)])
-def test_products_of_17_to_64_rows_in_tiles(ops, M, N, K):
+@pytest.mark.parametrize("M,N,K", [(17, 96, 256), (33, 1000, 512), (64, 4096, 1024), (48, 520, 768), (20, 64, 3072), (64, 12, 256),
+                                   (65, 200, 512), (96, 1000, 768), (100, 520, 1024), (128, 4096, 256), (81, 36, 1280)])
+def test_products_of_17_to_128_rows_in_tiles(ops, M, N, K):
     """The tile kernel behind `gemm_silu_mul` and `gemm_split`: every tile width (8, 6, 4 and 2 strips),
     plain, gated and with K cut into ranges, against the matrix product in float64; rows and columns that
     do not fill the last tile, chunk counts that are no multiple of three."""
