@@ -110,6 +110,20 @@ extern "C" int as_blas_adopt(int M, int N, int K, int out_dtype, size_t workspac
   return -1;
 }
 
+// The library builds its table of kernels by number at the first look-up (a third of a second here);
+// this makes that look-up, with the number of some candidate of some planned shape, so that a later
+// as_blas_adopt in the middle of serving does not pay for it.  Returns 1 if a look-up was made.
+extern "C" int as_blas_prepare_adoption() {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (auto& kept : g_plans) {
+    if (kept.second.candidates.empty()) continue;
+    std::vector<int> wanted = {hipblaslt_ext::getIndexFromAlgo(kept.second.candidates[0].algo)};
+    std::vector<hipblasLtMatmulHeuristicResult_t> found;
+    return ok(hipblaslt_ext::getAlgosFromIndex(g_handle, wanted, found)) ? 1 : 0;
+  }
+  return 0;
+}
+
 // Runs candidate `candidate` of the shape's plan.  a [M, K], w [N, K] bf16; out [M, N] bf16 or fp32;
 // workspace: device memory of at least workspace_bytes (the size the plan was made for).
 extern "C" int as_blas_gemm(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K, int candidate,

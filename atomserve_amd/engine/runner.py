@@ -315,6 +315,8 @@ class ModelRunner:
                 if not ops.library_trials_pending():
                     break
             ops.settle_library_choices()
+        if lengths:
+            ops.prepare_library_adoption()
         torch.cuda.synchronize()
         return lengths
 

@@ -37,6 +37,7 @@ SIGNATURES = {
     "as_blas_plan": ("blas", [I, I, I, I, c_size_t]),
     "as_blas_candidate_index": ("blas", [I, I, I, I, c_size_t, I]),
     "as_blas_adopt": ("blas", [I, I, I, I, c_size_t, I]),
+    "as_blas_prepare_adoption": ("blas", []),
     "as_blas_gemm": ("blas", [P, P, P, I, I, I, I, I, P, c_size_t, P]),
     "as_argmax": ("sampling", [P, P, I, I, P]),
     "as_sample": ("sampling", [P, I, I, P, P, P, P, P, P, P]),

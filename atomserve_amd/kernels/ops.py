@@ -498,6 +498,12 @@ def _choice_of_tuned_rows(M, N, K, dtype):
     return place if place >= 0 else 0
 
 
+def prepare_library_adoption() -> bool:
+    """Pays the library's one-time cost of finding a kernel by its number (a third of a second) now, not
+    at the first prompt of a length that was not tuned.  False while no shape has been planned."""
+    return bool(entry("as_blas_prepare_adoption")())
+
+
 def _library_call(a, w, out, M, N, K, candidate) -> None:
     call("as_blas_gemm", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, candidate,
          _ptr(_library["workspace"]), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip

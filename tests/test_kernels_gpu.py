@@ -414,6 +414,7 @@ def test_a_product_of_any_row_count_takes_what_the_tuned_count_above_it_chose(op
             ops._library_call(a1, w, o1, M + 1, N, K, place)
             assert close_bf16(o1, pk.gemm(a1, w), scale=math.sqrt(K)), place
         assert entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, -1) < 0
+        assert ops.prepare_library_adoption()  # the look-up by number that a warm-up makes ahead of serving
     finally:
         ops.LIBRARY_TUNED_ROWS.discard(tuned)
         ops.fix_library_choices(was_fixed)
