@@ -179,16 +179,17 @@ class Engine:
             self._thread = None
 
     def warm_up(self) -> int:
-        """Before serving: the decode steps of every batch size up to max_num_seqs are captured now
-        (kernels are compiled and loaded, the library's candidates tried) rather than at their
-        first use.  Returns the number of graphs captured; 0 where decode steps run uncaptured."""
+        """Before serving: the decode steps of every batch size up to max_num_seqs (and every context
+        length up to max_model_len, if that many graphs are kept) are captured now (kernels are compiled
+        and loaded, the library's candidates tried) rather than at their first use.  Returns the number
+        of graphs captured; 0 where decode steps run uncaptured."""
         tune = getattr(self.runner, "tune_prompt_lengths", None)
         if tune is not None:  # and the library's products of prompts of a few lengths, up to a step's budget
             tune(self.scheduler.config.max_num_batched_tokens)
         graphs = getattr(self.runner, "decode_graphs", None)
         if graphs is None:
             return 0
-        return graphs.capture_ahead(self.scheduler.config.max_num_seqs)
+        return graphs.capture_ahead(self.scheduler.config.max_num_seqs, self.scheduler.config.max_model_len)
 
     def profile_phases(self, on: bool = True):
         """Starts (or ends) the split of the host's time by phase; returns the `PhaseTimes` that

@@ -205,17 +205,24 @@ class DecodeGraphs:
         return held + sum(s["total_size"] for s in segments if tuple(s["segment_pool_id"]) == tuple(self.pool))
 
     @torch.inference_mode()
-    def capture_ahead(self, max_rows: int) -> int:
-        """Captures the decode step of every row bucket up to the one that holds `max_rows`, for the
-        first context bucket, with rows that store nothing: a server does this once at its start
-        instead of pausing when a bucket is first met.  Returns how many graphs were captured."""
+    def capture_ahead(self, max_rows: int, max_context: int = 0) -> int:
+        """Captures the decode step of every row bucket up to the one that holds `max_rows`, with rows that
+        store nothing: a server does this once at its start instead of pausing (for tens of milliseconds)
+        when a bucket is first met.  For every context bucket up to `max_context` if all of them fit among
+        the graphs that are kept, else for the first one only.  Returns how many graphs were captured."""
         if not self.eligible([self.filler()]):
             return 0
         before = len(self.graphs)
-        for n in self.ROW_BUCKETS:
-            self.run([self.filler() for _ in range(n)])
-            if n >= min(max_rows, self.most_rows):
-                break
+        most = min(max_rows, self.most_rows)
+        row_buckets = [n for n in self.ROW_BUCKETS if n < most] + [_bucket(most, self.ROW_BUCKETS)]
+        contexts = [self.CONTEXT_STEP * i for i in range(1, -(-max(max_context, 1) // self.CONTEXT_STEP) + 1)]
+        if len(contexts) * len(row_buckets) > self.MAX_GRAPHS:
+            contexts = contexts[:1]
+        bs = self.runner.manager.block_size
+        for context in contexts:
+            for n in row_buckets:
+                if (n, context) not in self.graphs:
+                    self.graphs[(n, context)] = self._capture(n, -(-context // bs), context)
         return len(self.graphs) - before
 
 

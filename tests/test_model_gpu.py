@@ -488,6 +488,13 @@ def test_a_step_sent_ahead_may_be_the_first_of_its_graph(tmp_path):
         logits_bytes = engine.runner.decode_graphs.most_rows * raw["vocab_size"] * 4
         assert engine.stats()["graph_bytes"] >= logits_bytes
     assert outs[0] == outs[1] and all(len(o) == 24 for o in outs[0])
+    # a warm-up captures both context lengths that max_model_len allows ahead: the same tokens from graphs
+    # that were captured on rows that only pad, and nothing is captured while the requests run
+    engine = create_engine(model, EngineConfig(block_size=16, num_blocks=160, max_model_len=1100, max_num_seqs=3,
+                                               max_num_batched_tokens=2048))  # fmt: skip
+    assert engine.warm_up() == 6
+    assert sorted(engine.runner.decode_graphs.graphs) == [(n, c) for n in (1, 2, 4) for c in (1024, 2048)]
+    assert engine.generate(prompts, params) == outs[0] and len(engine.runner.decode_graphs.graphs) == 6
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
