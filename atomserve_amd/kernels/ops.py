@@ -570,7 +570,7 @@ def _fastest_of(trial) -> int:
     return best
 
 
-# ---- 17 to 64 rows: tiles of weight rows with the activations staged in LDS ---------------------
+# ---- 17 to 64 (128) rows: tiles of weight rows with the activations staged in LDS ---------------
 # (the product cut along K, whose partial sums the next norm adds up, up to 128 rows: there the
 # library needs 42 us for Qwen3-8B's down projection and 21 for o, this kernel 24 on average; the
 # gated product of 96 and 128 rows is the library's with the activation after it, 48 and 56 us
