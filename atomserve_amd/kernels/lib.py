@@ -29,10 +29,11 @@ SIGNATURES = {
     "as_attn_decode_fresh": ("attention", [P, P, P, I, P, P, F, I, P, P, P, I, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
     "as_attn_prefill_mfma": ("attention", [P, P, P, P, I, P, I, P, I, I, I, I, F, I, P]),
     "as_gemm_f32": ("gemm", [P, P, P, I, I, I, P]),
-    "as_gemm_bf16_skinny": ("gemm", [P, P, P, I, I, I, I, I, P]),
-    "as_gemm_bf16_gated": ("gemm", [P, P, P, I, I, I, P]),
-    "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, I, I, I, P]),
-    "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, I, I, I, I, P]),
+    "as_gemm_bf16_skinny": ("gemm", [P, P, P, P, I, I, I, I, I, P]),
+    "as_gemm_bf16_gated": ("gemm", [P, P, P, P, I, I, I, P]),
+    "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, P, I, I, I, P]),
+    "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, P, I, I, I, I, P]),
+    "as_wave_order": ("gemm", [P, P, I, I, P]),
     "as_gemm_bf16_tile": ("gemm", [P, P, P, P, I, I, I, I, I, I, I, P]),
     "as_blas_plan": ("blas", [I, I, I, I, c_size_t]),
     "as_blas_candidate_index": ("blas", [I, I, I, I, c_size_t, I]),

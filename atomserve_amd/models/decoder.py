@@ -47,6 +47,7 @@ class DecoderModel:
         """Hand every part its tensors, by the names of `weight_decls`."""
         self.embed_weight = tensors["embed.weight"]
         self.head_weight = self.embed_weight if self.plan.tied_head else tensors["head.weight"]
+        ops.wave_order(self.head_weight)  # the head's product streams it at every decode step
         for i, block in enumerate(self.blocks):
             for part_name, part in block.parts().items():
                 prefix = f"layers.{i}.{part_name}."

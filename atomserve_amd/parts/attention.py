@@ -54,6 +54,11 @@ class Attention(Mixer):
             decls["k_norm.weight"] = WeightDecl((s.head_dim,), role="vector")
         return decls
 
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        for w in (self.qkv_weight, self.o_weight):
+            ops.wave_order(w)  # what the few-rows products of a decode step stream, where the sizes allow
+
     def cache_request(self):
         s = self.spec
         return PagedCacheRequest(s.num_kv_heads, s.head_dim, s.window)

@@ -24,6 +24,11 @@ class GatedMLP(FeedForward):
             "down.weight": WeightDecl((s.hidden_size, s.intermediate_size)),
         }
 
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        for w in (self.gate_up_weight, self.down_weight):
+            ops.wave_order(w)  # what the few-rows products of a decode step stream, where the sizes allow
+
     def forward(self, h, step, residual=None, next_norm=None):
         s, env = self.spec, self.env
         pending = isinstance(h, PendingNorm)

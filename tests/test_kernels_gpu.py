@@ -535,6 +535,55 @@ def test_gemm_scaled_bf16(ops, M, N, K, gated):
     assert bool(((out.double() - want).abs() <= bound).all())
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 96, 512), (8, 1024, 4096), (5, 4096, 1024), (16, 608, 2048), (3, 48, 6144), (8, 4096, 12288),
+                                   (13, 304, 6400), (16, 64, 8192), (32, 256, 1024), (20, 144, 2048), (17, 1024, 12288), (8, 32, 3072),
+                                   (7, 80, 5120), (8, 96, 64), (4, 64, 576), (8, 40, 512), (8, 48, 520)])  # fmt: skip
+def test_weights_in_wave_order_give_the_same_products(ops, M, N, K):
+    """The copy of a weight matrix in the order in which a wave reads it holds the same values at the places
+    the kernels' indexing says, and every few-rows product that finds such a copy on its weights gives bit for
+    bit what it gives from rows (the same values reach the same lanes).  Sizes of both few-rows kernels,
+    whole and partial workgroup rounds, one and two row tiles; sizes that take no copy go on as before."""
+    torch.manual_seed(M * 7 + N)
+    w = (torch.randn(2 * N, K, device=DEV) / math.sqrt(K)).to(BF16)
+    copy = ops.wave_order(w)
+    if (2 * N) % 16 or K % 64:
+        assert copy is None and not hasattr(w, ops.WAVE_ORDER)
+        return
+    want = w.view(2 * N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous().view(2 * N, K)  # strip, step, half, lane / 16, lane % 16
+    assert torch.equal(copy, want) and getattr(w, ops.WAVE_ORDER) is copy
+    plain = w.clone()  # the same values without a copy
+    a = torch.randn(M, K, device=DEV).to(BF16)
+
+    def both(run, *outs):
+        """run(weights, *outputs) with the copy and without: equal outputs."""
+        got = [o.clone() for o in outs]
+        run(w, *got)
+        ref = [o.clone() for o in outs]
+        run(plain, *ref)
+        for g, r in zip(got, ref):
+            assert torch.equal(g, r)
+        return got
+
+    for dtype in (BF16, F32):
+        if ops._few_rows(M, K, 2 * N):
+            both(lambda wt, out: ops.gemm(a, wt, out), torch.empty(M, 2 * N, dtype=dtype, device=DEV))
+    if ops._few_rows(M, K, N, ops.GATED_MAX_K) or ops._gated_two_tiles(M, K):
+        both(lambda wt, out: ops.gemm_silu_mul(a, wt, out), torch.empty(M, N, dtype=BF16, device=DEV))
+    if ops.gemm_link_supported(M, 2 * N, K, BF16):
+        gain = torch.randn(2 * N, device=DEV) * 0.3 + 1
+        x0 = torch.randn(M, 2 * N, device=DEV)
+        both(lambda wt, x, scaled, ssq: ops.gemm_link(a, wt, x, gain, scaled, ssq), x0,
+             torch.zeros(M, 2 * N, dtype=BF16, device=DEV), torch.zeros(M, 2 * N // 16, device=DEV))
+    if ops.gemm_link_supported(M, K, 8, BF16):
+        ssq = (a.float() ** 2).view(M, K // 16, 16).sum(-1).contiguous()
+        for gated in (False, True):
+            both(lambda wt, out: ops.gemm_scaled(a, ssq, 1e-5, wt, out, gated=gated),
+                 torch.empty(M, N if gated else 2 * N, dtype=BF16, device=DEV))
+    # a changed matrix takes a new copy; one that no longer qualifies loses it
+    w.mul_(2)
+    assert torch.equal(ops.wave_order(w), (want.float() * 2).to(BF16))
+
+
 def test_gemm_link_refuses_what_it_cannot_do(ops):
     assert not ops.gemm_link_supported(33, 1024, 1024, BF16)
     assert not ops.gemm_link_supported(32, 4096, 4096, BF16)  # two row tiles of such rows in 256 workgroups: more bytes than the weights
