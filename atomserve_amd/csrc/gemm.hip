@@ -612,7 +612,7 @@ constexpr int TILE_KC = 256;
 constexpr int tile_waves(int ns) { return ns == 6 ? 6 : 8; }
 constexpr int TILE_RING = 2;
 
-template <int MT, int NS, bool GATED, bool PARTIAL, typename OutT>
+template <int MT, int NS, bool GATED, bool PARTIAL, typename OutT, bool TILED = false>  // TILED: w in wave order (N % 16 == 0)
 __global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(const bf16* __restrict__ a,
                                                                         const bf16* __restrict__ w,
                                                                         OutT* __restrict__ out,
@@ -648,7 +648,13 @@ __global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(con
   const __amdgpu_buffer_rsrc_t a_buf = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<bf16*>(a), 0, (int)((unsigned)M * (unsigned)K * 2u), 0x00020000);
   constexpr unsigned BEYOND = 0xfffffff0u;
-  const unsigned w_off = (((unsigned)min(n0 + lr, N - 1) + (is_up ? (unsigned)N : 0u)) * (unsigned)K + k0 + lg * 16) * 2u;
+  // byte offset of this lane's first 16 bytes of the strip at k0: in its row, or (wave order) in the strip's run of
+  // 2 KB steps; a step of 64 columns further lies 128 bytes further in a row and 2 KB further in wave order, the
+  // second half of a lane's 32 bytes 16 bytes and 1 KB further
+  constexpr unsigned W_STEP = TILED ? 2048u : 128u, W_HALF = TILED ? 1024u : 16u, W_AUX = TILED ? 2 : 0;  // 2: non-temporal
+  const unsigned w_off =
+      TILED ? (((unsigned)(n0 >> 4) + (is_up ? (unsigned)(N >> 4) : 0u)) * (unsigned)(K >> 6) + (unsigned)(k0 >> 6)) * 2048u + lane * 16u
+            : (((unsigned)min(n0 + lr, N - 1) + (is_up ? (unsigned)N : 0u)) * (unsigned)K + k0 + lg * 16) * 2u;
 
   // ---- activations: chunk j travels through registers (requested one chunk ahead, 16-byte loads
   // spread over the threads) into LDS slot j % 2 just before it is used
@@ -680,12 +686,12 @@ __global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(con
   // roles rotate with the chunks (copying one set into another would wait for the newest loads).
   u32x4_t wa[STEPS][2], wb[STEPS][2], wc[STEPS][2];
   auto fetch = [&](u32x4_t (&into)[STEPS][2], int j) {
-    const unsigned base = j < nchunks ? w_off + where(j) * (TILE_KC * 2) : BEYOND;
+    const unsigned base = j < nchunks ? w_off + where(j) * (4 * W_STEP) : BEYOND;  // a chunk is four steps
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
-      const unsigned at = j < nchunks ? base + (kw + i * KW) * 128 : BEYOND;
-      into[i][0] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, at, 0, 0);
-      into[i][1] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, j < nchunks ? at + 16 : BEYOND, 0, 0);
+      const unsigned at = j < nchunks ? base + (kw + i * KW) * W_STEP : BEYOND;
+      into[i][0] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, at, 0, W_AUX);
+      into[i][1] = __builtin_amdgcn_raw_buffer_load_b128(w_buf, j < nchunks ? at + W_HALF : BEYOND, 0, W_AUX);
     }
   };
   floatx4 acc[MT];
@@ -772,30 +778,35 @@ __global__ __launch_bounds__(tile_waves(NS) * 64) void gemm_bf16_tile_kernel(con
 }
 
 template <int MT, int NS>
-static int launch_tile(const void* a, const void* w, void* out, float* partial, int out_dtype, int M, int N, int K,
-                       int gated, int splits, hipStream_t stream) {
+static int launch_tile(const void* a, const void* w, const void* wt, void* out, float* partial, int out_dtype, int M,
+                       int N, int K, int gated, int splits, hipStream_t stream) {
   constexpr int TILE_WAVES = tile_waves(NS);
   const size_t ring = (size_t)TILE_RING * MT * 16 * 32 * 16, meet = (size_t)TILE_WAVES * MT * 64 * 16;
   const size_t shmem = ring > meet ? ring : meet;
   const int k_per_split = K / (splits > 0 ? splits : 1);
   const int per_tile = 16 * (gated ? NS / 2 : NS);
   const dim3 grid((N + per_tile - 1) / per_tile, splits > 0 ? splits : 1);
-#define TILE_GO(GATEDV, PARTIALV, T)                                                                      \
+#define TILE_GO(GATEDV, PARTIALV, T, TILEDV)                                                              \
   do {                                                                                                    \
-    auto kernel = gemm_bf16_tile_kernel<MT, NS, GATEDV, PARTIALV, T>;                                     \
+    auto kernel = gemm_bf16_tile_kernel<MT, NS, GATEDV, PARTIALV, T, TILEDV>;                             \
     static bool raised = false;                                                                           \
     if (shmem > (48u << 10) && !raised) {                                                                 \
       if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,            \
                               (int)shmem) != hipSuccess) return AS_LAUNCH_FAILED;                         \
       raised = true;                                                                                      \
     }                                                                                                     \
-    kernel<<<grid, TILE_WAVES * 64, shmem, stream>>>((const bf16*)a, (const bf16*)w, (T*)out, partial,    \
+    kernel<<<grid, TILE_WAVES * 64, shmem, stream>>>((const bf16*)a, (const bf16*)(TILEDV ? wt : w), (T*)out, partial, \
                                                      M, N, K, k_per_split);                               \
   } while (0)
-  if (splits > 0) TILE_GO(false, true, float);
-  else if (gated && out_dtype == DT_BF16) TILE_GO(true, false, bf16);
-  else if (!gated && out_dtype == DT_BF16) TILE_GO(false, false, bf16);
-  else if (!gated && out_dtype == DT_F32) TILE_GO(false, false, float);
+  // the two variants that decode steps run also read weights in wave order
+  const bool tiled = takes_wave_order(wt, N, K);
+  if (splits > 0 && tiled && NS == 4) {  // the split products of the engine have tiles of four strips
+    if constexpr (NS == 4) TILE_GO(false, true, float, true);
+  } else if (splits > 0) TILE_GO(false, true, float, false);
+  else if (gated && out_dtype == DT_BF16 && tiled) TILE_GO(true, false, bf16, true);
+  else if (gated && out_dtype == DT_BF16) TILE_GO(true, false, bf16, false);
+  else if (!gated && out_dtype == DT_BF16) TILE_GO(false, false, bf16, false);
+  else if (!gated && out_dtype == DT_F32) TILE_GO(false, false, float, false);
   else return AS_BAD_DTYPE;
 #undef TILE_GO
   return launch_status();
@@ -807,8 +818,10 @@ static int launch_tile(const void* a, const void* w, void* out, float* partial, 
 //   splits > 0:  K is cut into `splits` ranges (each a multiple of 256) and the fp32 sums of every
 //                range go to partial[splits, M, N]; `out` is not written.
 //   strips:      weight rows per workgroup / 16: 8, 6, 4 or 2 (0: 8).
-extern "C" int as_gemm_bf16_tile(const void* a, const void* w, void* out, float* partial, int out_dtype, int M,
-                                 int N, int K, int gated, int splits, int strips, hipStream_t stream) {
+//   wt:          the weights in wave order or null; the gated and the split variant read them where N % 16 == 0.
+extern "C" int as_gemm_bf16_tile(const void* a, const void* w, const void* wt, void* out, float* partial,
+                                 int out_dtype, int M, int N, int K, int gated, int splits, int strips,
+                                 hipStream_t stream) {
   if (M <= 0) return AS_OK;
   if (M > 128 || N <= 0 || K <= 0 || (K % TILE_KC) || splits < 0) return AS_BAD_SHAPE;
   if (splits > 0 && (gated || !partial || (K % (splits * TILE_KC)))) return AS_BAD_SHAPE;
@@ -819,7 +832,7 @@ extern "C" int as_gemm_bf16_tile(const void* a, const void* w, void* out, float*
   int MT = (M + 15) / 16;
   if (MT > 4) MT = MT <= 6 ? 6 : 8;  // above 64 rows: tiles of 96 and 128 rows
 #define TILE_CASE(MTV, NSV) \
-  if (MT == MTV && strips == NSV) return launch_tile<MTV, NSV>(a, w, out, partial, out_dtype, M, N, K, gated, splits, stream)
+  if (MT == MTV && strips == NSV) return launch_tile<MTV, NSV>(a, w, wt, out, partial, out_dtype, M, N, K, gated, splits, stream)
   TILE_CASE(1, 8); TILE_CASE(2, 8); TILE_CASE(3, 8); TILE_CASE(4, 8);
   TILE_CASE(1, 6); TILE_CASE(2, 6); TILE_CASE(3, 6); TILE_CASE(4, 6);
   TILE_CASE(1, 4); TILE_CASE(2, 4); TILE_CASE(3, 4); TILE_CASE(4, 4);

@@ -34,7 +34,7 @@ SIGNATURES = {
     "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, P, I, I, I, P]),
     "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, P, I, I, I, I, P]),
     "as_wave_order": ("gemm", [P, P, I, I, P]),
-    "as_gemm_bf16_tile": ("gemm", [P, P, P, P, I, I, I, I, I, I, I, P]),
+    "as_gemm_bf16_tile": ("gemm", [P, P, P, P, P, I, I, I, I, I, I, I, P]),
     "as_blas_plan": ("blas", [I, I, I, I, c_size_t]),
     "as_blas_candidate_index": ("blas", [I, I, I, I, c_size_t, I]),
     "as_blas_adopt": ("blas", [I, I, I, I, c_size_t, I]),

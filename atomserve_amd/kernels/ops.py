@@ -651,7 +651,7 @@ def gemm_split(a, w, plan=None):
         raise KernelError(f"gemm_split: {M} rows, {K} -> {N} have no kernel")
     strips, splits = plan
     sums = torch.empty((splits, M, N), dtype=F32, device=a.device)
-    call("as_gemm_bf16_tile", _ptr(a), _ptr(w), 0, _ptr(sums), _DT[F32], M, N, K, 0, splits, strips, _stream())
+    call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _wave_ptr(w), 0, _ptr(sums), _DT[F32], M, N, K, 0, splits, strips, _stream())
     return sums
 
 
@@ -682,7 +682,7 @@ def gemm_silu_mul(a, w, out) -> None:
         call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), M, inter, K, _stream())
         return
     if _tile_rows(M, K, a.dtype):
-        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0,
+        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0,
              _gated_tile_strips(M, inter), _stream())  # fmt: skip
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)

@@ -1000,7 +1000,8 @@ def test_sampling_is_seeded_per_request_and_mixes_greedy_rows(ops):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 96, 256), (33, 1000, 512), (64, 4096, 1024), (48, 520, 768), (20, 64, 3072), (64, 12, 256),
-                                   (65, 200, 512), (96, 1000, 768), (100, 520, 1024), (128, 4096, 256), (81, 36, 1280)])
+                                   (65, 200, 512), (96, 1000, 768), (100, 520, 1024), (128, 4096, 256), (81, 36, 1280), (80, 160, 512),
+                                   (33, 48, 1024)])  # fmt: skip
 def test_products_of_17_to_128_rows_in_tiles(ops, M, N, K):
     """The tile kernel behind `gemm_silu_mul` and `gemm_split`: every tile width (8, 6, 4 and 2 strips),
     plain, gated and with K cut into ranges, against the matrix product in float64; rows and columns that
@@ -1014,22 +1015,23 @@ def test_products_of_17_to_128_rows_in_tiles(ops, M, N, K):
     ref = a.double() @ w.double().T
     gated_ref = (lambda g: torch.nn.functional.silu(g[:, :N]) * g[:, N:])(ref.to(BF16).double())
     chunks = K // 256
-    for strips in (8, 6, 4, 2):
+    copy = ops.wave_order(w) if N % 16 == 0 else None  # the gated and the split variant also read weights in wave order
+    for strips, wt in [(n, p) for n in (8, 6, 4, 2) for p in ([0] if copy is None else [0, copy.data_ptr()])]:
         out = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
-        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), out.data_ptr(), 0, 1, M, N, K, 0, 0, strips, stream)
+        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, out.data_ptr(), 0, 1, M, N, K, 0, 0, strips, stream)
         assert close_bf16(out, ref[:, :N]), f"plain, {strips} strips"
         out32 = torch.full((M, N), float("nan"), dtype=F32, device=DEV)
-        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), out32.data_ptr(), 0, 0, M, N, K, 0, 0, strips, stream)
+        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, out32.data_ptr(), 0, 0, M, N, K, 0, 0, strips, stream)
         assert torch.allclose(out32.double(), ref[:, :N], atol=1e-3, rtol=1e-4)
         out.fill_(float("nan"))
-        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), out.data_ptr(), 0, 1, M, N, K, 1, 0, strips, stream)
+        call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, out.data_ptr(), 0, 1, M, N, K, 1, 0, strips, stream)
         # a sum that rounds to the neighbouring bfloat16 moves the activation by a step of its input
         assert torch.allclose(out.double(), gated_ref, atol=2e-2, rtol=2e-2), f"gated, {strips} strips"
         for splits in {1, chunks, max(1, chunks // 2)}:
             if chunks % splits:
                 continue
             sums = torch.full((splits, M, N), float("nan"), dtype=F32, device=DEV)
-            call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), 0, sums.data_ptr(), 0, M, N, K, 0, splits, strips, stream)
+            call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, 0, sums.data_ptr(), 0, M, N, K, 0, splits, strips, stream)
             assert torch.allclose(sums.double().sum(0), ref[:, :N], atol=1e-3, rtol=1e-4), f"{splits} ranges, {strips} strips"
     # through the wrappers: the gated product, and split sums taken in by the norm
     act = torch.empty(M, N, dtype=BF16, device=DEV)
