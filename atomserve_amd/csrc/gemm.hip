@@ -805,7 +805,9 @@ static int launch_tile(const void* a, const void* w, const void* wt, void* out, 
   } else if (splits > 0) TILE_GO(false, true, float, false);
   else if (gated && out_dtype == DT_BF16 && tiled) TILE_GO(true, false, bf16, true);
   else if (gated && out_dtype == DT_BF16) TILE_GO(true, false, bf16, false);
-  else if (!gated && out_dtype == DT_BF16) TILE_GO(false, false, bf16, false);
+  else if (!gated && out_dtype == DT_BF16 && tiled && NS <= 4) {  // narrow tiles: what a plain product of few columns takes
+    if constexpr (NS <= 4) TILE_GO(false, false, bf16, true);
+  } else if (!gated && out_dtype == DT_BF16) TILE_GO(false, false, bf16, false);
   else if (!gated && out_dtype == DT_F32) TILE_GO(false, false, float, false);
   else return AS_BAD_DTYPE;
 #undef TILE_GO
@@ -818,7 +820,8 @@ static int launch_tile(const void* a, const void* w, const void* wt, void* out, 
 //   splits > 0:  K is cut into `splits` ranges (each a multiple of 256) and the fp32 sums of every
 //                range go to partial[splits, M, N]; `out` is not written.
 //   strips:      weight rows per workgroup / 16: 8, 6, 4 or 2 (0: 8).
-//   wt:          the weights in wave order or null; the gated and the split variant read them where N % 16 == 0.
+//   wt:          the weights in wave order or null; read where N % 16 == 0 by the gated variant, the split variant
+//                (tiles of 4 strips) and the plain bf16 variant (tiles of 2 and 4 strips).
 extern "C" int as_gemm_bf16_tile(const void* a, const void* w, const void* wt, void* out, float* partial,
                                  int out_dtype, int M, int N, int K, int gated, int splits, int strips,
                                  hipStream_t stream) {

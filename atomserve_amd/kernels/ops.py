@@ -463,7 +463,8 @@ def library_choices_fixed() -> bool:
 
 def library_choices() -> dict:
     """(rows, columns, width, output dtype) -> the candidate that runs, for every shape settled so far
-    (-1: torch's own call); enough to reproduce a run's products."""
+    (-1: torch's own call; OWN_CANDIDATE + strips: this package's tile product); enough to reproduce a
+    run's products."""
     return dict(_library["choice"])
 
 
@@ -489,7 +490,7 @@ def _library_gemm(a, w, out, M, N, K) -> None:
             count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
             if count == 0:
                 choice = state["choice"][key] = -1  # the library offers nothing for this shape through this door
-            elif count == 1 or state["fixed"]:
+            elif state["fixed"] or (count == 1 and not _own_candidates(M, N, K, out.dtype, w)):
                 choice = state["choice"][key] = 0  # the library's first candidate, which is what torch.mm runs
             elif M not in LIBRARY_TUNED_ROWS:
                 choice = _choice_of_tuned_rows(M, N, K, out.dtype)  # a prompt of any length: what its bucket settled on
@@ -498,7 +499,8 @@ def _library_gemm(a, w, out, M, N, K) -> None:
                 else:
                     state["choice"][key] = choice
             else:
-                trial = state["trials"][key] = {"count": count, "runs": []}
+                ids = list(range(count)) + _own_candidates(M, N, K, out.dtype, w)
+                trial = state["trials"][key] = {"count": len(ids), "ids": ids, "runs": []}
         if trial is not None:
             if not capturing and not _tried_enough(trial):
                 trial["last"] = (a, w, out)
@@ -507,6 +509,8 @@ def _library_gemm(a, w, out, M, N, K) -> None:
             choice = state["choice"][key] = _fastest_of(state["trials"].pop(key))
     if choice < 0:
         return _torch_gemm(a, w, out)
+    if choice >= OWN_CANDIDATE and not _wave_ptr(w):
+        choice = 0  # chosen on weights that had a copy in wave order; these have none
     _library_call(a, w, out, M, N, K, choice)
 
 
@@ -523,6 +527,8 @@ def _choice_of_tuned_rows(M, N, K, dtype):
         return None
     if settled < 0:
         return 0
+    if settled >= OWN_CANDIDATE:  # this package's tile kernel: for this row count too if it takes it, else the library's first
+        return settled if settled in _own_candidates(M, N, K, dtype, None) else 0
     index = entry("as_blas_candidate_index")(tuned, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, settled)
     place = entry("as_blas_adopt")(M, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, index)
     return place if place >= 0 else 0
@@ -534,7 +540,30 @@ def prepare_library_adoption() -> bool:
     return bool(entry("as_blas_prepare_adoption")())
 
 
+# Beside the library's candidates a trial may time this package's plain tile product (17 to 128 rows, K in
+# chunks of 256, bf16 out, weights with a copy in wave order) with tiles of 2 and of 4 strips: for qkv
+# of Qwen3-8B sizes it takes 12.7 / 14.8 / 16.3 us at 32 / 48 / 64 rows against the library's best 14.7 /
+# 17.3 / 17.6; for the 4,096 columns of o the library wins at 32 to 64 rows.  Such a candidate's number
+# is OWN_CANDIDATE + its strips.
+OWN_CANDIDATE = 1000
+
+
+def _own_candidates(M, N, K, dtype, w) -> list:
+    """w: the weights, to see whether they have a copy in wave order; None: taken for granted."""
+    if dtype != BF16 or not _tile_rows(M, K, BF16, TILE_SPLIT_MAX_ROWS) or N % 16:
+        return []
+    if w is not None and not _wave_ptr(w):
+        return []
+    return [OWN_CANDIDATE + 2, OWN_CANDIDATE + 4]
+
+
 def _library_call(a, w, out, M, N, K, candidate) -> None:
+    if candidate >= OWN_CANDIDATE:
+        if not _wave_ptr(w) or out.dtype != BF16:
+            raise KernelError("the tile product was chosen for weights with a copy in wave order and bf16 results")
+        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), 0, _DT[BF16], M, N, K, 0, 0,
+             candidate - OWN_CANDIDATE, _stream())  # fmt: skip
+        return
     call("as_blas_gemm", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, candidate,
          _ptr(_library["workspace"]), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip
 
@@ -545,7 +574,7 @@ def _tried_enough(trial) -> bool:
 
 def _trial_run(trial, a, w, out, M, N, K) -> None:
     """Computes the product with the candidate whose turn it is, between two events."""
-    candidate = len(trial["runs"]) % trial["count"]
+    candidate = trial["ids"][len(trial["runs"]) % trial["count"]]
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     try:

@@ -420,6 +420,43 @@ def test_a_product_of_any_row_count_takes_what_the_tuned_count_above_it_chose(op
         ops.fix_library_choices(was_fixed)
 
 
+def test_the_tile_product_is_a_candidate_beside_the_librarys(ops):
+    """For 17 to 128 rows and weights with a copy in wave order, a trial also times this package's plain tile
+    product (tiles of 2 and 4 strips); chosen, it gives the product, and weights without a copy fall back
+    to the library's first candidate under the same choice."""
+    torch.manual_seed(5)
+    M, N, K = 48, 544, 1024
+    a = torch.randn(M, K, device=DEV).to(BF16)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(BF16)
+    bare = w.clone()
+    assert ops._own_candidates(M, N, K, BF16, w) == []  # no copy yet
+    ops.wave_order(w)
+    own = ops._own_candidates(M, N, K, BF16, w)
+    assert own == [ops.OWN_CANDIDATE + 2, ops.OWN_CANDIDATE + 4]
+    assert ops._own_candidates(M, N + 8, K, BF16, None) == [] and ops._own_candidates(16, N, K, BF16, None) == []
+    assert ops._own_candidates(M, N, K + 64, BF16, None) == [] and ops._own_candidates(129, N, K, BF16, None) == []
+    ref = pk.gemm(a, w)
+    key = (M, N, K, BF16)
+    kept = ops._library["choice"].get(key)
+    try:
+        for candidate in own:
+            out = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
+            ops._library_call(a, w, out, M, N, K, candidate)
+            assert close_bf16(out, ref, scale=1.0)
+            ops._library_gemm(a, w, out, M, N, K)  # makes the library's plan and workspace for this shape
+            ops._library["choice"][key] = candidate
+            for weights in (w, bare):
+                out.fill_(float("nan"))
+                ops._library_gemm(a, weights, out, M, N, K)
+                assert close_bf16(out, ref, scale=1.0)
+    finally:
+        ops._library["trials"].pop(key, None)
+        if kept is None:
+            ops._library["choice"].pop(key, None)
+        else:
+            ops._library["choice"][key] = kept
+
+
 def test_library_candidates_replay_from_a_graph(ops):
     """Each candidate captured once and replayed with other inputs and a workspace full of noise,
     with eager work and synchronisations between the replays: every replay gives what the eager
