@@ -629,12 +629,12 @@ def _fastest_of(trial) -> int:
     return best
 
 
-# ---- 17 to 64 (128) rows: tiles of weight rows with the activations staged in LDS ---------------
-# (the product cut along K, whose partial sums the next norm adds up, up to 128 rows: there the
-# library needs 42 us for Qwen3-8B's down projection and 21 for o, this kernel 24 on average; the
-# gated product of 96 and 128 rows is the library's with the activation after it, 48 and 56 us
-# against 51 and 61)
-TILE_MAX_ROWS = 64
+# ---- 17 to 128 rows: tiles of weight rows with the activations staged in LDS --------------------
+# (above 64 rows in row tiles of 96 and 128.  At 128 rows the library needs 42 us for Qwen3-8B's down
+# projection and 21 for o, the split product 24 on average; the gated product of 96 and 128 rows lost to
+# the library's with the activation after it while it read the weights from rows, 51 and 61 us against
+# 48 and 56, and wins by a little since it reads them in wave order: batch 96 9,507 -> 9,587 tokens/s)
+TILE_MAX_ROWS = 128
 TILE_SPLIT_MAX_ROWS = 128
 TILE_CHUNK = 256  # K comes in chunks of this many
 
