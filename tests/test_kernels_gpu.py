@@ -604,8 +604,15 @@ def test_weights_in_wave_order_give_the_same_products(ops, M, N, K):
     for dtype in (BF16, F32):
         if ops._few_rows(M, K, 2 * N):
             both(lambda wt, out: ops.gemm(a, wt, out), torch.empty(M, 2 * N, dtype=dtype, device=DEV))
-    if ops._few_rows(M, K, N, ops.GATED_MAX_K) or ops._gated_two_tiles(M, K):
+    if ops._few_rows(M, K, N, ops.GATED_MAX_K):
         both(lambda wt, out: ops.gemm_silu_mul(a, wt, out), torch.empty(M, N, dtype=BF16, device=DEV))
+    elif ops._gated_two_tiles(M, K, plain):
+        # 17 to 32 wide rows: from rows the persistent kernel with two row tiles, with the copy the tile product
+        assert not ops._gated_two_tiles(M, K, w)
+        with_copy, from_rows = torch.empty(M, N, dtype=BF16, device=DEV), torch.empty(M, N, dtype=BF16, device=DEV)
+        ops.gemm_silu_mul(a, w, with_copy)
+        ops.gemm_silu_mul(a, plain, from_rows)
+        assert torch.allclose(with_copy.float(), from_rows.float(), atol=2e-2, rtol=2e-2)
     if ops.gemm_link_supported(M, 2 * N, K, BF16):
         gain = torch.randn(2 * N, device=DEV) * 0.3 + 1
         x0 = torch.randn(M, 2 * N, device=DEV)
