@@ -40,7 +40,7 @@ class RMSNorm(Norm):
 
     def absorb(self, a, w, x):
         M, N = x.shape
-        if not ops.gemm_link_supported(M, N, a.shape[1], self.env.dtype):
+        if not ops.gemm_link_supported(M, N, a.shape[1], self.env.dtype, w):
             return None
         scaled = torch.empty((M, N), dtype=self.env.dtype, device=x.device)
         ssq = torch.empty((M, -(-N // 16)), dtype=torch.float32, device=x.device)

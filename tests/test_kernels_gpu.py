@@ -602,12 +602,18 @@ def test_weights_in_wave_order_give_the_same_products(ops, M, N, K):
         return got
 
     for dtype in (BF16, F32):
-        if ops._few_rows(M, K, 2 * N):
+        if ops._few_rows(M, K, 2 * N, w=w):
             both(lambda wt, out: ops.gemm(a, wt, out), torch.empty(M, 2 * N, dtype=dtype, device=DEV))
-    if ops._few_rows(M, K, N, ops.GATED_MAX_K):
+        elif ops._few_rows(M, K, 2 * N) and dtype == BF16:
+            # 17 to 32 rows: from rows the persistent kernel with two row tiles, with the copy the tile products or the library
+            with_copy, from_rows = torch.empty(M, 2 * N, dtype=BF16, device=DEV), torch.empty(M, 2 * N, dtype=BF16, device=DEV)
+            ops.gemm(a, w, with_copy)
+            ops.gemm(a, plain, from_rows)
+            assert close_bf16(with_copy, from_rows.double(), scale=1.0)
+    if ops._few_rows(M, K, N, ops.GATED_MAX_K, w=w):
         both(lambda wt, out: ops.gemm_silu_mul(a, wt, out), torch.empty(M, N, dtype=BF16, device=DEV))
-    elif ops._gated_two_tiles(M, K, plain):
-        # 17 to 32 wide rows: from rows the persistent kernel with two row tiles, with the copy the tile product
+    elif ops._few_rows(M, K, N, ops.GATED_MAX_K) or ops._gated_two_tiles(M, K, plain):
+        # 17 to 32 rows: from rows the persistent kernel with two row tiles, with the copy the tile product
         assert not ops._gated_two_tiles(M, K, w)
         with_copy, from_rows = torch.empty(M, N, dtype=BF16, device=DEV), torch.empty(M, N, dtype=BF16, device=DEV)
         ops.gemm_silu_mul(a, w, with_copy)
