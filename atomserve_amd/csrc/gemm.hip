@@ -368,10 +368,10 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
                                                                                OutT* __restrict__ out, int M, int N,
                                                                                int K, int nstrips,
                                                                                NormLink link = NormLink{}) {
-  static_assert(NST % 2 == 0, "a wave's slice is handled in two halves");
+  static_assert(NST >= 2, "a wave's slice is handled in two halves");
   static_assert(!TILED || !MASKED, "weights in wave order come in whole steps");
   static_assert(!LINK || (!GATED && !SCALED && sizeof(OutT) == 4), "the stream is fp32 and takes a plain product");
-  constexpr int H = NST / 2;
+  constexpr int H = (NST + 1) / 2, H2 = NST - H;  // steps of the first and of the second half
   __shared__ floatx4 red[2][MT][PIPE_WAVES * 64];
   __shared__ float inv_rms[16 * MT];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -384,8 +384,8 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
   if (strip >= nstrips) return;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 #define PIPE_VALID(U, HALF) (!MASKED || kbase + (U) * 64 + (HALF) * 8 + 8 <= K)
-#define PIPE_LOAD(BUF, ROW, OFF)                                                                              \
-  _Pragma("unroll") for (int u = 0; u < H; ++u) {                                                             \
+#define PIPE_LOAD(BUF, ROW, OFF, CNT)                                                                         \
+  _Pragma("unroll") for (int u = 0; u < CNT; ++u) {                                                           \
     if constexpr (TILED) {                                                                                    \
       BUF[u][0] = WAVE_ORDER16(ROW + ((OFF) + u) * 1024);                                                     \
       BUF[u][1] = WAVE_ORDER16(ROW + ((OFF) + u) * 1024 + 512);                                               \
@@ -394,8 +394,8 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
       BUF[u][1] = PIPE_VALID((OFF) + u, 1) ? *reinterpret_cast<const bf16x8*>(ROW + ((OFF) + u) * 64 + 8) : zero; \
     }                                                                                                         \
   }
-#define PIPE_MATH(BUF, OFF)                                                                                   \
-  _Pragma("unroll") for (int u = 0; u < H; ++u) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {             \
+#define PIPE_MATH(BUF, OFF, CNT)                                                                              \
+  _Pragma("unroll") for (int u = 0; u < CNT; ++u) _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {           \
     acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][0], av[mt][(OFF) + u][0], acc[mt], 0, 0, 0);       \
     acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(BUF[u][1], av[mt][(OFF) + u][1], acc[mt], 0, 0, 0);       \
   }
@@ -403,10 +403,10 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
 #define PIPE_ROWS(STRIP, UP)                                                                                          \
   (TILED ? w + (((size_t)(STRIP) + ((UP) ? (size_t)(N >> 4) : 0)) * (K >> 6) + wave * NST) * 1024 + lane * 8          \
          : w + ((size_t)min((STRIP) * 16 + lr, N - 1) + ((UP) ? (size_t)N : 0)) * K + kbase)
-  bf16x8 w0[H][2], w1[H][2];
+  bf16x8 w0[H][2], w1[H2][2];
   const bf16* wrow = PIPE_ROWS(strip, false);
-  PIPE_LOAD(w0, wrow, 0)
-  PIPE_LOAD(w1, wrow, H)
+  PIPE_LOAD(w0, wrow, 0, H)
+  PIPE_LOAD(w1, wrow, H, H2)
   bf16x8 av[MT][NST][2];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -441,10 +441,10 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
     floatx4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    PIPE_MATH(w0, 0)
-    if (more) { PIPE_LOAD(w0, nrow, 0) }
-    PIPE_MATH(w1, H)
-    if (more) { PIPE_LOAD(w1, nrow, H) }
+    PIPE_MATH(w0, 0, H)
+    if (more) { PIPE_LOAD(w0, nrow, 0, H) }
+    PIPE_MATH(w1, H, H2)
+    if (more) { PIPE_LOAD(w1, nrow, H, H2) }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) red[buf][mt][wave * 64 + lane] = acc[mt];
     __syncthreads();
@@ -516,11 +516,13 @@ template <bool GATED, typename OutT, bool SCALED = false, bool LINK = false>
 static int dispatch_pipe(const void* a, const void* w, const void* wt, void* out, int M, int N, int K,
                          hipStream_t stream, const NormLink& link = NormLink{}) {
   if (!pipe_fits(M, K)) return AS_BAD_SHAPE;
-  const int nst = 2 * ((K + 128 * PIPE_WAVES - 1) / (128 * PIPE_WAVES));
+  int nst = 2 * ((K + 128 * PIPE_WAVES - 1) / (128 * PIPE_WAVES));
+  if (K > 64 * PIPE_WAVES * 4 && K <= 64 * PIPE_WAVES * 5) nst = 5;  // a width of 2,560 (Qwen3-4B) in five whole steps a wave, not six masked ones
   if (M > 16) {
     switch (nst) {
       case 2: return launch_pipe<2, GATED, OutT, SCALED, LINK, 2>(a, w, wt, out, M, N, K, link, stream);
       case 4: return launch_pipe<4, GATED, OutT, SCALED, LINK, 2>(a, w, wt, out, M, N, K, link, stream);
+      case 5: return launch_pipe<5, GATED, OutT, SCALED, LINK, 2>(a, w, wt, out, M, N, K, link, stream);
       case 6: return launch_pipe<6, GATED, OutT, SCALED, LINK, 2>(a, w, wt, out, M, N, K, link, stream);
       case 8: return launch_pipe<8, GATED, OutT, SCALED, LINK, 2>(a, w, wt, out, M, N, K, link, stream);
     }
@@ -529,6 +531,7 @@ static int dispatch_pipe(const void* a, const void* w, const void* wt, void* out
   switch (nst) {
     case 2: return launch_pipe<2, GATED, OutT, SCALED, LINK, 1>(a, w, wt, out, M, N, K, link, stream);
     case 4: return launch_pipe<4, GATED, OutT, SCALED, LINK, 1>(a, w, wt, out, M, N, K, link, stream);
+    case 5: return launch_pipe<5, GATED, OutT, SCALED, LINK, 1>(a, w, wt, out, M, N, K, link, stream);
     case 6: return launch_pipe<6, GATED, OutT, SCALED, LINK, 1>(a, w, wt, out, M, N, K, link, stream);
     case 8: return launch_pipe<8, GATED, OutT, SCALED, LINK, 1>(a, w, wt, out, M, N, K, link, stream);
     case 10: return launch_pipe<10, GATED, OutT, SCALED, LINK, 1>(a, w, wt, out, M, N, K, link, stream);

@@ -35,6 +35,15 @@ SIZES = {
     "32b": dict(vocab_size=151936, hidden_size=5120, intermediate_size=25600, num_layers=64, num_heads=64,
                 num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
                 max_position_embeddings=40960),
+    "1.7b": dict(vocab_size=151936, hidden_size=2048, intermediate_size=6144, num_layers=28, num_heads=16,
+                 num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True,
+                 max_position_embeddings=40960),
+    "4b": dict(vocab_size=151936, hidden_size=2560, intermediate_size=9728, num_layers=36, num_heads=32,
+               num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True,
+               max_position_embeddings=40960),
+    "14b": dict(vocab_size=151936, hidden_size=5120, intermediate_size=17408, num_layers=40, num_heads=40,
+                num_kv_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
+                max_position_embeddings=40960),
 }  # fmt: skip
 
 
@@ -47,7 +56,7 @@ def parse_args():
     p.add_argument("--context", type=int, default=2048)
     p.add_argument("--shortest-context", type=int, default=0, help="contexts spread evenly from this many tokens to "
                    "--context over the batch instead of all equal (0: equal)")
-    p.add_argument("--sizes", choices=sorted(SIZES), default="8b", help="layer sizes of Qwen3-8B, -0.6B or -32B")
+    p.add_argument("--sizes", choices=sorted(SIZES), default="8b", help="layer sizes of a dense Qwen3 model")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both counts are reported)")
     p.add_argument("--max-len", type=int, default=4096, help="longest sequence the cache pool is sized for")
     p.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")

@@ -294,7 +294,7 @@ def test_gemm_fp32_rows_do_not_depend_on_the_batch(ops):
                                    (4, 1040, 5120), (7, 520, 6144), (2, 100, 2560), (11, 4100, 3072), (8, 512, 12288),
                                    (13, 300, 6152), (17, 300, 4096), (32, 6144, 1024), (25, 1000, 1000),
                                    (31, 520, 3072), (20, 64, 4096), (32, 300, 24), (32, 6144, 4096), (8, 6150, 4096), (1, 10240, 2048),
-                                   (24, 6147, 1024)])  # fmt: skip
+                                   (24, 6147, 1024), (9, 304, 2304), (16, 6144, 2560), (20, 96, 2560)])  # fmt: skip
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(8)
     a, w = torch.randn(M, K, device=DEV).to(BF16), torch.randn(N, K, device=DEV).to(BF16)
@@ -310,7 +310,7 @@ def test_gemm_bf16(ops, M, N, K):
 @pytest.mark.parametrize("M,I,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 12288, 4096), (9, 700, 2048),
                                    (3, 40, 200), (16, 24, 8), (4, 520, 5120), (7, 264, 6144), (8, 128, 12288),
                                    (40, 300, 512), (32, 1030, 2048), (17, 264, 2048), (29, 128, 4096),
-                                   (24, 72, 200), (32, 12288, 4096), (20, 3000, 4096)])  # fmt: skip
+                                   (24, 72, 200), (32, 12288, 4096), (20, 3000, 4096), (8, 9728, 2560), (6, 200, 2312)])  # fmt: skip
 def test_gemm_silu_mul_bf16(ops, M, I, K):
     """Gate and up products with the activation in one kernel (few rows, an input that fits)
     or as product then activation: the same numbers as the two kernels give, which are the plain
@@ -504,7 +504,8 @@ def test_gemm_silu_mul_fp32(ops):
 
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1032, 4096), (16, 4096, 4096), (3, 40, 200),
                                    (16, 24, 8), (8, 520, 12288), (13, 304, 6152), (4, 4096, 6144), (32, 1024, 4096),
-                                   (17, 1032, 12288), (27, 520, 200), (32, 2048, 4104), (20, 40, 2048)])  # fmt: skip
+                                   (17, 1032, 12288), (27, 520, 200), (32, 2048, 4104), (20, 40, 2048), (8, 2560, 2560),
+                                   (12, 2560, 9728)])  # fmt: skip
 def test_gemm_link_bf16(ops, M, N, K):
     """The product that adds into the fp32 stream and prepares the next norm: the stream receives
     exactly the product kernel's bf16 output; beside it x * gain rounded to bf16 and the sums of
@@ -534,7 +535,8 @@ def test_gemm_link_bf16(ops, M, N, K):
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (8, 1000, 96), (5, 1030, 4096), (16, 6144, 4096), (9, 700, 2048),
                                    (3, 40, 200), (16, 24, 8), (7, 264, 3072), (2, 130, 5120), (32, 6144, 1024),
-                                   (17, 1030, 2048), (26, 40, 200), (31, 264, 2048), (6, 6148, 4096), (20, 6144, 2048)])  # fmt: skip
+                                   (17, 1030, 2048), (26, 40, 200), (31, 264, 2048), (6, 6148, 4096), (20, 6144, 2048),
+                                   (8, 6144, 2560), (3, 100, 2400)])  # fmt: skip
 def test_gemm_scaled_bf16(ops, M, N, K, gated):
     """The product that finishes a pending norm: x * gain arrives rounded to bf16, 1 / rms comes
     from the sums of squares and multiplies the fp32 sums.  That input times the plain 1 / rms is
@@ -574,7 +576,8 @@ def test_gemm_scaled_bf16(ops, M, N, K, gated):
 
 @pytest.mark.parametrize("M,N,K", [(1, 96, 512), (8, 1024, 4096), (5, 4096, 1024), (16, 608, 2048), (3, 48, 6144), (8, 4096, 12288),
                                    (13, 304, 6400), (16, 64, 8192), (32, 256, 1024), (20, 144, 2048), (17, 1024, 12288), (8, 32, 3072),
-                                   (7, 80, 5120), (8, 96, 64), (4, 64, 576), (8, 40, 512), (8, 48, 520)])  # fmt: skip
+                                   (7, 80, 5120), (8, 96, 64), (4, 64, 576), (8, 40, 512), (8, 48, 520), (8, 512, 2560),
+                                   (16, 9728, 2560), (8, 2560, 9728)])  # fmt: skip
 def test_weights_in_wave_order_give_the_same_products(ops, M, N, K):
     """The copy of a weight matrix in the order in which a wave reads it holds the same values at the places
     the kernels' indexing says, and every few-rows product that finds such a copy on its weights gives bit for
