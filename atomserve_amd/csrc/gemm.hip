@@ -786,7 +786,8 @@ static int launch_tile(const void* a, const void* w, const void* wt, void* out, 
   constexpr int TILE_WAVES = tile_waves(NS);
   const size_t ring = (size_t)TILE_RING * MT * 16 * 32 * 16, meet = (size_t)TILE_WAVES * MT * 64 * 16;
   const size_t shmem = ring > meet ? ring : meet;
-  const int k_per_split = K / (splits > 0 ? splits : 1);
+  // ranges of whole chunks, the last one possibly shorter
+  const int k_per_split = splits > 0 ? (K / TILE_KC + splits - 1) / splits * TILE_KC : K;
   const int per_tile = 16 * (gated ? NS / 2 : NS);
   const dim3 grid((N + per_tile - 1) / per_tile, splits > 0 ? splits : 1);
 #define TILE_GO(GATEDV, PARTIALV, T, TILEDV)                                                              \
@@ -820,8 +821,9 @@ static int launch_tile(const void* a, const void* w, const void* wt, void* out, 
 // out[M, N] = a[M, K] @ w[N, K]^T for 1 <= M <= 128 and K % 256 == 0 through the tile kernel
 // (row tiles of 16 up to 64 rows, 96 or 128 rows above; two chunks of 128 rows take 128 KB of LDS).
 //   gated != 0:  w is [2 N, K] (gate rows, then up rows), out[M, N] = silu(gate) * up, bf16.
-//   splits > 0:  K is cut into `splits` ranges (each a multiple of 256) and the fp32 sums of every
-//                range go to partial[splits, M, N]; `out` is not written.
+//   splits > 0:  K is cut into `splits` ranges of ceil(K / 256 / splits) chunks of 256 (the last range may be
+//                shorter, none may be empty) and the fp32 sums of every range go to partial[splits, M, N];
+//                `out` is not written.
 //   strips:      weight rows per workgroup / 16: 8, 6, 4 or 2 (0: 8).
 //   wt:          the weights in wave order or null; read where N % 16 == 0 by the gated variant, the split variant
 //                (tiles of 4 strips) and the plain bf16 variant (tiles of 2 and 4 strips).
@@ -830,7 +832,10 @@ extern "C" int as_gemm_bf16_tile(const void* a, const void* w, const void* wt, v
                                  hipStream_t stream) {
   if (M <= 0) return AS_OK;
   if (M > 128 || N <= 0 || K <= 0 || (K % TILE_KC) || splits < 0) return AS_BAD_SHAPE;
-  if (splits > 0 && (gated || !partial || (K % (splits * TILE_KC)))) return AS_BAD_SHAPE;
+  if (splits > 0) {  // every range gets at least one chunk
+    const int chunks = K / TILE_KC, per = (chunks + splits - 1) / splits;
+    if (gated || !partial || (long long)(splits - 1) * per >= chunks) return AS_BAD_SHAPE;
+  }
   if (splits == 0 && !out) return AS_BAD_SHAPE;
   if (strips == 0) strips = 8;
   if (strips != 8 && strips != 6 && strips != 4 && strips != 2) return AS_BAD_SHAPE;

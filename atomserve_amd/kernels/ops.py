@@ -660,16 +660,16 @@ def _gated_tile_strips(rows: int, outputs: int) -> int:
 
 def gemm_split_plan(rows: int, n: int, k: int, dtype):
     """(strips, splits) of `gemm_split` for a product of these sizes, or None where it has no kernel:
-    tiles of 64 weight rows, and K cut into as many ranges (of whole chunks) as fill the compute
-    units with those tiles."""
+    tiles of 64 weight rows, and K cut into as many ranges (of whole chunks, as equal as they come) as
+    fill the compute units with those tiles."""
     if not _tile_rows(rows, k, dtype, TILE_SPLIT_MAX_ROWS) or n % 4:
         return None
     strips = 4
     tiles = -(-n // (16 * strips))
     chunks = k // TILE_CHUNK
-    want = max(1, compute_units() // tiles)
-    splits = max(d for d in range(1, chunks + 1) if chunks % d == 0 and d <= want)
-    return strips, splits
+    want = max(1, min(chunks, compute_units() // tiles))
+    per = -(-chunks // want)  # chunks of a range; the last range may have fewer (38 chunks in 6 ranges: 7, 7, 7, 7, 7, 3)
+    return strips, -(-chunks // per)
 
 
 def gemm_split(a, w, plan=None):

@@ -1080,11 +1080,16 @@ def test_products_of_17_to_128_rows_in_tiles(ops, M, N, K):
         call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, out.data_ptr(), 0, 1, M, N, K, 1, 0, strips, stream)
         # a sum that rounds to the neighbouring bfloat16 moves the activation by a step of its input
         assert torch.allclose(out.double(), gated_ref, atol=2e-2, rtol=2e-2), f"gated, {strips} strips"
-        for splits in {1, chunks, max(1, chunks // 2)}:
-            if chunks % splits:
+        for splits in sorted({1, 2, 3, chunks, max(1, chunks // 2), max(1, chunks - 1)}):
+            if splits > chunks:
                 continue
             sums = torch.full((splits, M, N), float("nan"), dtype=F32, device=DEV)
-            call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, 0, sums.data_ptr(), 0, M, N, K, 0, splits, strips, stream)
+            run = lambda: call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, 0, sums.data_ptr(), 0, M, N, K, 0, splits, strips, stream)
+            if (splits - 1) * -(-chunks // splits) >= chunks:  # ranges of ceil(chunks / splits) chunks would leave the last ones empty
+                with pytest.raises(ops.KernelError):
+                    run()
+                continue
+            run()  # ranges of equal length, or the last one shorter
             assert torch.allclose(sums.double().sum(0), ref[:, :N], atol=1e-3, rtol=1e-4), f"{splits} ranges, {strips} strips"
     # through the wrappers: the gated product, and split sums taken in by the norm
     act = torch.empty(M, N, dtype=BF16, device=DEV)
