@@ -667,7 +667,7 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 // s_waitcnt that only constrains the vector-memory counter (vmcnt: bits 3:0 and 15:14)
 #define PF_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-template <int DC>
+template <int DC, int QT>  // D / 32; column tiles of 16 queries that a wave owns: 2, or 1 (see the launcher)
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ tiles, const int* __restrict__ block_tables, int table_width,
@@ -703,30 +703,31 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
 
   // the keys this workgroup walks: from the first key any of its waves sees to the last
   int wg_lo = 0x7fffffff, wg_last = -1;
-  for (int u = bz * 4; u < bz * 4 + 4 && u < 2 * G; ++u) {
-    const int uq0 = (u / G) * 32;
+  constexpr int WQ = 16 * QT, PARTS = 64 / WQ;  // queries of a wave; waves that share a head's 64 queries
+  for (int u = bz * 4; u < bz * 4 + 4 && u < PARTS * G; ++u) {
+    const int uq0 = (u / G) * WQ;
     if (uq0 >= count) continue;
-    wg_last = max(wg_last, pos0 + min(count, uq0 + 32) - 1);
+    wg_last = max(wg_last, pos0 + min(count, uq0 + WQ) - 1);
     wg_lo = min(wg_lo, window > 0 ? max(0, pos0 + uq0 - window + 1) : 0);
   }
   if (wg_last < 0) return;  // uniform over the workgroup
 
   // this wave's queries
   const int unit = bz * 4 + wave;
-  const int half = unit / G, head = kvh * G + unit % G;
-  const int q0 = half * 32;
-  const bool working = unit < 2 * G && q0 < count;
-  const int nq = working ? min(32, count - q0) : 1;
+  const int head = kvh * G + unit % G;
+  const int q0 = (unit / G) * WQ;
+  const bool working = unit < PARTS * G && q0 < count;
+  const int nq = working ? min(WQ, count - q0) : 1;
   const int my_last = working ? pos0 + q0 + nq - 1 : -1;
   const int my_first_q = pos0 + q0;                  // position of this wave's first query
   const float scale2 = scale * 1.4426950408889634f;  // scores are kept in base 2
   const int my_lo = working ? (window > 0 ? max(0, pos0 + q0 - window + 1) : 0) : 0x7fffffff;
 
-  bf16x8_t qop[2][DC];
-  int qpos[2];
-  bool qok[2];
+  bf16x8_t qop[QT][DC];
+  int qpos[QT];
+  bool qok[QT];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     const int qi = qt * 16 + col;
     qok[qt] = working && qi < nq;
     const int qc = min(qi, nq - 1);  // columns past the end repeat the last query and are not stored
@@ -740,10 +741,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       for (int c = 0; c < DC; ++c) qop[qt][c] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
   }
-  f32x4_t o[2][DT];
-  float m[2], l[2];
+  f32x4_t o[QT][DT];
+  float m[QT], l[QT];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     m[qt] = NEG_INF;
     l[qt] = 0.f;
 #pragma unroll
@@ -851,10 +852,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       }
     }
     if (active) {
-      // raw scores of 64 keys x 32 queries; a key operand is read from LDS once for both query tiles
-      f32x4_t sc[2][4];
+      // raw scores of 64 keys x 16 QT queries; a key operand is read from LDS once for all of a wave's query tiles
+      f32x4_t sc[QT][4];
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt)
+      for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) sc[qt][tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       // The operands of a whole tile are asked from LDS before its products start, and the next
@@ -875,7 +876,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
         for (int c = 0; c < DC; ++c) {
           const bf16x8_t kop = __builtin_bit_cast(bf16x8_t, kraw[tt & 1][c]);
 #pragma unroll
-          for (int qt = 0; qt < 2; ++qt)
+          for (int qt = 0; qt < QT; ++qt)
             sc[qt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[qt][c], sc[qt][tt], 0, 0, 0);
         }
         if (more) {  // a quarter of the round's copies behind each tile's products
@@ -886,11 +887,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       // Only rounds that touch the causal diagonal, the window's edge or the end of the context
       // need a mask; the others see all 64 keys (uniform over the wave).
       const bool masked = kb + 63 > my_first_q || (window > 0 && kb < my_last - window + 1);
-      bf16x8_t pop[2][2];
-      float alpha[2];
+      bf16x8_t pop[QT][2];
+      float alpha[QT];
       bool rescale = false;
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
+      for (int qt = 0; qt < QT; ++qt) {
         if (masked) {
 #pragma unroll
           for (int tt = 0; tt < 4; ++tt)
@@ -931,7 +932,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       // first keys have been seen)
       if (__any(rescale)) {
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
+        for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha[qt];
       }
@@ -951,14 +952,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt) {
           const bf16x8_t vop = __builtin_bit_cast(bf16x8_t, vraw[j][dt]);
 #pragma unroll
-          for (int qt = 0; qt < 2; ++qt) o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt][j], o[qt][dt], 0, 0, 0);
+          for (int qt = 0; qt < QT; ++qt) o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop, pop[qt][j], o[qt][dt], 0, 0, 0);
         }
       }
     }
   }
 
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     if (!qok[qt]) continue;
     const float inv = 1.0f / l[qt];
     bf16* orow = out + ((size_t)(tok0 + q0 + qt * 16 + col) * H + head) * D + 4 * grp;
@@ -973,19 +974,30 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
 
 // tiles: [num_tiles, 4] int32 (first flat token, count <= 64, block-table row, first position);
 // fastest when sorted by first position + count, largest first.
+// query_tiles: 2, a wave owns 32 queries of a head and a workgroup two heads' 64; or 1, a wave owns 16 and a
+// workgroup one head's 64: twice the workgroups, each with half the arithmetic for the same keys and values
+// brought into LDS, so that a round of 64 keys is shorter.  That pays where few work items decide the time
+// (a lone prompt of a few thousand tokens: its last tile's rounds are a chain that nothing shortens).
 extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, const int* tiles,
                                     int num_tiles, const int* block_tables, int table_width, void* out, int H,
-                                    int KV, int D, int bs, float scale, int window, hipStream_t stream) {
+                                    int KV, int D, int bs, float scale, int window, int query_tiles,
+                                    hipStream_t stream) {
   if (num_tiles <= 0) return AS_OK;
   if (H <= 0 || KV <= 0 || H % KV || bs <= 0 || table_width <= 0) return AS_BAD_SHAPE;
   const int G = H / KV;
   if (D % 32 || D <= 0 || D > 256 || bs % 16) return AS_BAD_SHAPE;
-  const int units_z = (2 * G + 3) / 4;
+  if (query_tiles != 1 && query_tiles != 2) return AS_BAD_SHAPE;
+  const int units_z = (64 / (16 * query_tiles) * G + 3) / 4;
   const long items = (long)num_tiles * KV * units_z;
   if (items > 0x7fffffffL) return AS_BAD_SHAPE;
   const int pass = compute_units();
 #define LAUNCH(DCV)                                                                                   \
-  attn_prefill_mfma_kernel<DCV><<<(int)items, 256, 0, stream>>>(                                      \
+  if (query_tiles == 1)                                                                               \
+    attn_prefill_mfma_kernel<DCV, 1><<<(int)items, 256, 0, stream>>>(                                 \
+        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, tiles, block_tables, table_width, \
+        (bf16*)out, H, KV, bs, scale, window, units_z, pass);                                         \
+  else                                                                                                \
+  attn_prefill_mfma_kernel<DCV, 2><<<(int)items, 256, 0, stream>>>(                                   \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, tiles, block_tables, table_width,   \
       (bf16*)out, H, KV, bs, scale, window, units_z, pass)
   switch (D / 32) {

@@ -357,12 +357,27 @@ def attn_prefill_supported(dtype, head_dim: int, block_size: int) -> bool:
     return dtype == BF16 and head_dim % 32 == 0 and head_dim <= PREFILL_MAX_HEAD_DIM and block_size % 16 == 0
 
 
-def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context) -> None:
+# The prefill attention has two variants: a wave owns 32 queries of a head (two column tiles of 16), four waves two
+# heads' 64 queries; or a wave owns 16 and four waves one head's 64, which makes twice the workgroups with half the
+# arithmetic each for the same keys and values brought into LDS.  The second pays while the first would give a
+# compute unit one workgroup at most (a 2,048-token prompt of Qwen3-0.6B sizes 6.24 -> 5.79 ms, 8,192 tokens 30.96 ->
+# 28.27 ms, 512 tokens of Qwen3-8B sizes 11.26 -> 10.92 ms); beyond that it loses (2,048 tokens of Qwen3-8B
+# sizes 28.18 -> 28.28 ms, 16,384 tokens 297.6 -> 323.2 ms).
+PREFILL_QUERY_TILES = None  # 1 or 2 to force a variant (measurements); None: chosen by the sizes
+
+
+def _prefill_query_tiles(num_tiles: int, H: int, KV: int) -> int:
+    return 1 if num_tiles * KV * -(-2 * (H // KV) // 4) <= compute_units() else 2
+
+
+
+def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context, query_tiles=None) -> None:
     """Causal attention of prompt portions over the paged cache, bfloat16, on the matrix cores.
 
     tiles [Nt, 4] int32: (first flat token, count <= 64, block-table row, position of the first
     token) of up to 64 consecutive tokens of one request; the keys of these tokens are already in
-    the pages.  max_context: host bound on the last position + 1 of any tile."""
+    the pages.  max_context: host bound on the last position + 1 of any tile.
+    query_tiles: column tiles of 16 queries that a wave owns, 2 or 1; None: chosen here."""
     _check(q, "q", BF16, (None, None, None))
     T, H, D = q.shape
     _check(out, "out", BF16, (T, H, D))
@@ -377,8 +392,11 @@ def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, m
         raise KernelError(f"prefill attention: unsupported heads {H}/{KV}, head width {D} or page size {bs}")
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
+    if query_tiles is None:
+        query_tiles = PREFILL_QUERY_TILES or _prefill_query_tiles(tiles.shape[0], H, KV)
     call("as_attn_prefill_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(tiles), tiles.shape[0],
-         _ptr(block_tables), block_tables.shape[1], _ptr(out), H, KV, D, bs, float(scale), int(window), _stream())  # fmt: skip
+         _ptr(block_tables), block_tables.shape[1], _ptr(out), H, KV, D, bs, float(scale), int(window),
+         int(query_tiles), _stream())  # fmt: skip
 
 
 SKINNY_MAX_ROWS = 16  # up to here the bf16 product streams the weights through our own kernel

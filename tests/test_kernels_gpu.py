@@ -896,10 +896,11 @@ def test_attention_prefill(ops, H, KV, D, bs, window):
         for q0 in range(0, n, 64):
             tiles.append([flat + q0, min(64, n - q0), r, start + q0])
         flat += n
-    out = torch.zeros(T, H, D, dtype=BF16, device=DEV)
-    ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, window, max(lens))
     ref = pk.paged_attention(q, k_pages, v_pages, i32(list(range(T))), i32(positions), i32(tok_row), tables, D**-0.5, window)
-    assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), (out.float() - ref).abs().max()
+    for query_tiles in (None, 1, 2):  # as the sizes choose; a wave owning 16 queries; 32
+        out = torch.zeros(T, H, D, dtype=BF16, device=DEV)
+        ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, window, max(lens), query_tiles=query_tiles)
+        assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), (query_tiles, (out.float() - ref).abs().max())
 
 
 def test_attention_prefill_of_a_long_prompt_in_one_step(ops):
@@ -910,11 +911,12 @@ def test_attention_prefill_of_a_long_prompt_in_one_step(ops):
     _, k_pages, v_pages, tables, _ = paged_case(BF16, H, KV, D, bs, [start + n], seed=9, k_scale=2.0 / math.sqrt(D / 16))
     q = torch.randn(n, H, D, device=DEV).to(BF16)
     tiles = sorted(([q0, min(64, n - q0), 0, start + q0] for q0 in range(0, n, 64)), key=lambda t: -(t[3] + t[1]))
-    out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
-    ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, 0, start + n)
     check = list(range(0, n, 97)) + [n - 1]
     ref = pk.paged_attention(q, k_pages, v_pages, i32(check), i32(list(range(start, start + n))), i32([0] * n), tables, D**-0.5)
-    assert torch.allclose(out[check].float(), ref[check], atol=2e-2, rtol=2e-2), (out[check].float() - ref[check]).abs().max()
+    for query_tiles in (2, 1):
+        out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
+        ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, 0, start + n, query_tiles=query_tiles)
+        assert torch.allclose(out[check].float(), ref[check], atol=2e-2, rtol=2e-2), (out[check].float() - ref[check]).abs().max()
 
 
 def test_attention_prefill_sees_a_far_key_and_not_the_future(ops):
@@ -927,9 +929,10 @@ def test_attention_prefill_sees_a_far_key_and_not_the_future(ops):
         fut_page, fut_off = int(tables[0, 651 // bs]), 651 % bs
         k_pages[fut_page, 0, fut_off] = (q[650, 0].float() * 8.0).to(BF16)  # a stronger match, one step in the future
         tiles = [[q0, min(64, n - q0), 0, q0] for q0 in range(0, n, 64)]
-        out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
-        ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, 1.0, 0, n)
-        assert torch.allclose(out[650, 0].float(), v_pages[page, 0, :, off].float(), atol=2e-2), far
+        for query_tiles in (1, 2):
+            out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
+            ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, 1.0, 0, n, query_tiles=query_tiles)
+            assert torch.allclose(out[650, 0].float(), v_pages[page, 0, :, off].float(), atol=2e-2), (far, query_tiles)
 
 
 def test_kernels_refuse_what_they_cannot_do(ops):
