@@ -314,13 +314,20 @@ __device__ __forceinline__ void load_kv_step(KVStep<DC>& st, const bf16* __restr
   }
   {  // values: keys 8 grp .. 8 grp + 7 of coordinates col, col + 16, ...  One instruction of the wave reads two runs of
      // 512 bytes, every 128-byte line whole, and a decode step reads a value once: marked as not to be kept (batch 64
-     // of Qwen3-8B sizes 8,542 -> 8,872 tokens/s).  The keys' loads share their lines in pairs and stay as they are.
+     // of Qwen3-8B sizes 8,542 -> 8,872 tokens/s).  With pages of more than 32 tokens a step's 32 keys are part of a line,
+     // which the next step needs again: no mark there.  The keys' loads share their lines in pairs and stay as they are.
     const int pc = grp >> 1;
     const bool live = kb + 16 * pc < end;
     const bf16* vcol = v_pages + (pc ? head[1] : head[0]) + (pc ? off0[1] : off0[0]) + 8 * (grp & 1) + (size_t)col * bs;
+    if (bs <= 32) {  // uniform over the grid: two loops, so that neither holds a choice per load
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      st.v[dt] = live ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(vcol + (size_t)dt * 16 * bs)) : zero;
+      for (int dt = 0; dt < DT; ++dt)
+        st.v[dt] = live ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(vcol + (size_t)dt * 16 * bs)) : zero;
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        st.v[dt] = live ? *reinterpret_cast<const bf16x8_t*>(vcol + (size_t)dt * 16 * bs) : zero;
+    }
   }
 }
 
