@@ -415,14 +415,16 @@ def _workgroups() -> int:
 def _few_rows(rows: int, k: int, n: int, max_k=None, w=None) -> bool:
     """Whether a product of `rows` rows of width `k` with `n` output columns goes through the
     few-rows kernels of this package.  w: the weights, if known: with a copy in wave order, 17 to 32
-    rows are left to the tile products (and the library), which are then the faster ones also for narrow
-    rows (Qwen3-0.6B sizes, batch 32: 12,430 -> 12,580 to 12,750 tokens/s)."""
+    rows are left to the tile products (and the library), which are then the faster ones, also for narrow
+    rows (Qwen3-0.6B sizes, batch 32: 12,430 -> 12,580 to 12,750 tokens/s), and so are 9 to 16 rows of a
+    model that is wide enough (`_tile_preferred`; Qwen3-8B sizes, batch 16: 3,497 -> 3,594, batch 9: 2,045
+    -> 2,106; at 8 rows and fewer the few-rows kernels win: 2,129 against 2,019)."""
     if rows <= 0 or k % 8:
+        return False
+    if w is not None and _tile_preferred(rows, k, n, w):
         return False
     if rows <= SKINNY_MAX_ROWS:
         return max_k is None or k <= max_k
-    if w is not None and _wave_ptr(w) and _tile_rows(rows, k, BF16):
-        return False
     strips = min(-(-n // 16), _workgroups())
     return (rows <= SKINNY_TWO_MAX_ROWS and k <= SKINNY_TWO_MAX_K
             and strips * rows * k * 2 <= SKINNY_TWO_MAX_ACT_BYTES)  # fmt: skip
@@ -444,7 +446,7 @@ def gemm(a, w, out) -> None:
         return
     if out.dtype not in (BF16, F32):
         raise KernelError(f"gemm: unsupported output dtype {out.dtype}")
-    if _few_rows(M, K, N, w=w):
+    if _few_rows(M, K, N, w=w if out.dtype == BF16 else None):  # fp32 results (the head): no tile product to prefer
         call("as_gemm_bf16_skinny", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), _DT[out.dtype], M, N, K, 0, _stream())
     else:
         _library_gemm(a, w, out, M, N, K)
@@ -661,8 +663,24 @@ TILE_SPLIT_MAX_ROWS = 128
 TILE_CHUNK = 256  # K comes in chunks of this many
 
 
+TILE_MIN_ROWS = 9  # up to 8 rows the few-rows kernels are the faster ones in any case (one row tile of 16, half of it padding)
+# ... and at 9 to 16 rows while the model is narrow: with their residual sum and norm folded in they save two
+# launches a layer, which a small model's step is made of (decode at batch 16, tile products from 9 rows against
+# from 17: Qwen3-0.6B sizes 8,391 against 9,082 tokens/s, -1.7B 7,030 against 7,311, -4B 4,697 against 4,499,
+# -8B 3,594 against 3,497, -14B 2,311 against 2,069)
+TILE_FROM_9_MIN_WIDTH = 2560
+
+
 def _tile_rows(rows: int, k: int, dtype, most: int = TILE_MAX_ROWS) -> bool:
-    return dtype == BF16 and SKINNY_MAX_ROWS < rows <= most and k % TILE_CHUNK == 0
+    return dtype == BF16 and TILE_MIN_ROWS <= rows <= most and k % TILE_CHUNK == 0
+
+
+def _tile_preferred(rows: int, k: int, n: int, w) -> bool:
+    """Whether a product of 9 to 32 rows that the few-rows kernels could take is left to the tile products
+    (and the library with them as candidates): weights with a copy in wave order, a K in whole chunks, and
+    above 16 rows or a model wide enough (the narrower of k and n is the stream's width in all four
+    products of a layer)."""
+    return bool(_wave_ptr(w)) and _tile_rows(rows, k, BF16) and (rows > SKINNY_MAX_ROWS or min(k, n) >= TILE_FROM_9_MIN_WIDTH)
 
 
 def _gated_tile_strips(rows: int, outputs: int) -> int:
@@ -747,10 +765,10 @@ def gemm_link_supported(rows: int, n_out: int, k: int, dtype, w=None) -> bool:
     producer's weights, if known (see `_few_rows`)."""
     if dtype != BF16 or rows <= 0 or k % 8 or n_out % 8 or n_out > GATED_MAX_K:
         return False
+    if w is not None and _tile_preferred(rows, k, n_out, w):
+        return False
     if rows <= SKINNY_MAX_ROWS:
         return True
-    if w is not None and _wave_ptr(w) and _tile_rows(rows, k, BF16):
-        return False
     # two row tiles: the producer reads its activations once per strip of 16 outputs (whole rows
     # for every workgroup of the persistent kernel, and for every strip beyond its K), the consumer
     # keeps rows of n_out in registers in each of its workgroups
