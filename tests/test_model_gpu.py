@@ -294,18 +294,26 @@ def test_captured_steps_are_dropped_and_captured_again(setup):
     check(float((seen[True][-1][5] - ref).abs().max()), float(ref.abs().max()), "float32")
 
 
-def test_decode_graphs_at_real_layer_sizes(tmp_path_factory):
-    """The same at Qwen3-8B's layer sizes, where the products of 17 to 64 rows are the library's
-    with the candidate that the warm-up's trials chose: replays of the captured steps give what
-    eager steps give, replay after replay, and what the plain model gives."""
-    from atomserve_amd.weights.loader import load_model
-
+@pytest.fixture(scope="module")
+def like_8b(tmp_path_factory):
     raw = {**TINY_B_LIKE_8B}
     weights = plain_random_weights(raw, seed=78, std=0.02, gain_std=0.1)
-    path = write_model_dir(str(tmp_path_factory.mktemp("real_graphs")), raw, weights, torch.bfloat16)
-    model, _, _ = load_model(path, torch.bfloat16, "cuda:0")
-    for num_requests in (21, 40):
-        graphs_against_eager(model, raw, weights, "bfloat16", num_requests, torch.float32)
+    return raw, weights, write_model_dir(str(tmp_path_factory.mktemp("real_graphs")), raw, weights, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype,counts", [("bfloat16", (3, 9, 13, 16, 21, 40)), ("float32", (9, 16))])
+def test_decode_graphs_at_real_layer_sizes(like_8b, dtype, counts):
+    """The same at Qwen3-8B's layer sizes, where the row count of a decode step chooses its matrix products:
+    up to 8 rows the few-rows kernels with the residual sum and the norm folded in, 9 to 16 rows the tile
+    products with one row tile (split sums into the norm, the gated tile), 17 to 64 rows those with more
+    row tiles or the library's with the candidate that the warm-up's trials chose.  Replays of the captured
+    steps give what eager steps give, replay after replay, and what the plain model gives."""
+    from atomserve_amd.weights.loader import load_model
+
+    raw, weights, path = like_8b
+    model, _, _ = load_model(path, getattr(torch, dtype), "cuda:0")
+    for num_requests in counts:
+        graphs_against_eager(model, raw, weights, dtype, num_requests, torch.float32)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
