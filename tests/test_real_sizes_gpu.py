@@ -8,6 +8,7 @@ import random
 import pytest
 import torch
 
+import bench
 from tests import plain_qwen3 as plain
 from tests import replay_cases as rc
 
@@ -135,10 +136,11 @@ def wanted_rows(replay, steps):
 
 
 def test_the_mixed_batch_of_qwen3_06b_sizes_in_32_bit():
-    """The continuous batch of the benchmark, smaller: 12 requests with prompts of 64 to 1,024 tokens,
-    half of them sharing their first 32, a budget of 512 tokens a step, 24 tokens decoded each, greedy,
-    through scheduler, prefix cache and step function in 32-bit.  Every generated token is the plain
-    model's best at its place (the plain model sees prompt and reply whole, once per request)."""
+    """The continuous batch of the benchmark at its stated size: 32 requests with prompts of 64 to 2,048
+    tokens, half of them sharing their first 32, a budget of 512 tokens a step, 128 tokens decoded each,
+    greedy, through scheduler, prefix cache and step function in 32-bit (the analogue of reference
+    tests/test_engine.py:106-138 on random weights).  Every generated token is the plain model's best at
+    its place (the plain model sees prompt and reply whole, once per request, in float64 on the GPU)."""
     from atomserve_amd.config import EngineConfig
     from atomserve_amd.engine.engine import create_engine
     from atomserve_amd.engine.sequence import SamplingParams
@@ -147,21 +149,108 @@ def test_the_mixed_batch_of_qwen3_06b_sizes_in_32_bit():
     arch, config, stored, exact = device_weights(raw, seed=6)
     model = build(arch, config, exact, torch.float32)
     rng = random.Random(0)
+    requests, longest, decoded, budget, block = 32, 2048, 128, 512, 16
     prefix = [rng.randrange(raw["vocab_size"]) for _ in range(32)]
     prompts = []
-    for i in range(12):
-        body = [rng.randrange(raw["vocab_size"]) for _ in range(rng.randint(64, 1024))]
+    for i in range(requests):
+        body = [rng.randrange(raw["vocab_size"]) for _ in range(rng.randint(64, longest))]
         prompts.append(prefix + body[32:] if i % 2 == 0 else body)
-    decoded = 24
-    engine = create_engine(model, EngineConfig(block_size=16, num_blocks=6 * 1100 // 16, max_num_seqs=8,
-                                               max_num_batched_tokens=512, max_model_len=1100))  # fmt: skip
+    max_len = longest + decoded + block
+    engine = create_engine(model, EngineConfig(block_size=block, num_blocks=requests * max_len // block, max_num_seqs=requests,
+                                               max_num_batched_tokens=budget, max_model_len=max_len))  # fmt: skip
     outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=decoded, ignore_eos=True))
     stats = engine.stats()
-    assert stats["cached_prompt_tokens"] >= 5 * 32 and stats["kv_blocks_used"] == 0
+    assert stats["cached_prompt_tokens"] >= 15 * 32 and stats["kv_blocks_used"] == 0
+    assert stats["steps"] >= sum(map(len, prompts)) // budget + decoded - 1  # the prompts came in portions beside decoded tokens
+    del engine, model
+    torch.cuda.empty_cache()
+    exact64 = {k: v.double() for k, v in exact.items()}
     for p, out in zip(prompts, outs):
         assert len(out) == decoded
-        ref = plain.logits(raw, exact, p + out, **PLAIN)[len(p) - 1 : -1]
+        hidden = plain.hidden_states(raw, exact64, p + out, **PLAIN)[len(p) - 1 : -1]  # the places that chose the reply
+        ref = plain.rms_norm(hidden, exact64["model.norm.weight"], raw["rms_norm_eps"]) @ exact64["model.embed_tokens.weight"].T
         best = ref.max(dim=-1).values
         chosen = ref.gather(1, torch.tensor(out, device=ref.device)[:, None])[:, 0]
         # the token is the best one, or ties with it within 32-bit rounding of the logits
         assert float((best - chosen).max()) <= 2e-5 * float(ref.abs().max())
+
+
+def trace_of_every_route(vocab):
+    """Sixty-four short requests and a longer one: their prompts in one step (1,200 rows of the matrix
+    products), a portion of 5 tokens beside 64 decoded tokens, a portion of 65 tokens alone (a product of
+    65 rows), then decode steps of 64, 32, 16, 12, 8, 3 and 1 rows, two of each, as requests end: every
+    way a step's row count chooses the kernels of its matrix products and its attention."""
+    rng = random.Random(vocab)
+    requests = {f"r{i}": rc.random_ids(vocab, rng.randint(2, 36) + 15, seed=7000 + i) for i in range(64)}
+    requests["a"] = rc.random_ids(vocab, 140, seed=6999)
+    at = {rid: len(ids) - 15 for rid, ids in requests.items()}
+    at["a"] = 70
+    steps = [{"step": 0, "end": [], "entries": [{"id": rid, "tokens": ids[: at[rid]], "want": [at[rid] - 1]}
+                                                 for rid, ids in requests.items()]}]  # fmt: skip
+    alive = [f"r{i}" for i in range(64)]
+
+    def decode(rows, extra=(), end=()):
+        entries = list(extra)
+        for rid in alive[:rows]:
+            entries.append({"id": rid, "tokens": [requests[rid][at[rid]]], "want": [0]})
+            at[rid] += 1
+        steps.append({"step": len(steps), "entries": entries, "end": list(end)})
+
+    decode(64, extra=[{"id": "a", "tokens": requests["a"][70:75], "want": [0, 4]}])
+    steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": requests["a"][75:140], "want": [0, 33, 64]}], "end": ["a"]})
+    for rows in (64, 32, 16, 12, 8, 3, 1):
+        decode(rows)
+        decode(rows)
+    steps[-1]["end"] = alive
+    return requests, steps
+
+
+@pytest.mark.parametrize("dtype,products", [("float32", "first"), ("bfloat16", "first"), ("bfloat16", "timed")])
+@pytest.mark.parametrize("size", ["0.6b", "1.7b", "4b", "8b", "14b", "32b"])
+def test_layer_sizes_of_every_model_the_benchmark_names(size, dtype, products):
+    """Two layers of each dense Qwen3 model's sizes that `bench.py` names (widths of 1,024 to 5,120, 16 to 64
+    heads in groups of 2 to 8, feed-forwards of 3,072 to 25,600, tied and untied heads over a small vocabulary):
+    the sizes choose the kernels (steps a wave of the few-rows products, how K is cut for the split tile product,
+    the group of heads that one tile of the decode attention holds), and so do the rows of a step.  Every wanted
+    row of a trace that takes each route against the plain model in float64 on the GPU; in bfloat16 with the
+    library's first candidates and with the candidates (this package's tile products among them) that timing
+    picks, as serving does."""
+    from atomserve_amd.config import Qwen3Config
+    from atomserve_amd.engine.replay import Replay
+    from atomserve_amd.kernels import ops
+
+    assert set(bench.SIZES) == {"0.6b", "1.7b", "4b", "8b", "14b", "32b"}  # a size added there is added here
+    raw = Qwen3Config(**{**bench.SIZES[size], "num_layers": 2, "vocab_size": 5008}).to_dict()
+    arch, config, stored, exact = device_weights(raw, seed=17)
+    exact64 = {k: v.double() for k, v in exact.items()}
+    requests, steps = trace_of_every_route(raw["vocab_size"])
+    model = build(arch, config, exact if dtype == "float32" else stored, getattr(torch, dtype))
+    was_fixed = ops.library_choices_fixed()
+    try:
+        replay = Replay(None, dtype, rc.live_token_bound(steps), max_live=65, model=model, fixed_products=products == "first")
+        got = wanted_rows(replay, steps)
+        if products == "timed":  # the captured steps of 32 and 64 rows did settle on candidates of their own
+            assert {rows for rows, _, _, _ in ops.library_choices()} >= {32, 64} and not ops.library_trials_pending()
+    finally:
+        ops.fix_library_choices(was_fixed)
+    assert replay.manager.num_free == replay.manager.num_blocks and len(got) == 65 + 66 + 3 + 2 * (64 + 32 + 16 + 12 + 8 + 3 + 1)
+    assert sorted(n for n, _ in replay.runner.decode_graphs.graphs) == [1, 4, 8, 16, 32, 64]
+    err, noise, scale = Spread(), Spread(), 0.0
+    logits = {}
+    for rid, place, row in got:
+        if rid not in logits:
+            both = [plain.logits(raw, exact64, requests[rid], **PLAIN).float().cpu()]
+            if dtype == "bfloat16":
+                both.append(plain.logits(raw, exact64, requests[rid], storage=torch.bfloat16, **PLAIN).float().cpu())
+            logits[rid] = both
+        want = logits[rid][0][place]
+        err.add(row - want)
+        scale = max(scale, float(want.abs().max()))
+        if dtype == "bfloat16":
+            noise.add(logits[rid][1][place] - want)
+    print(f"{size} {dtype} {products}: |logits| {scale:.3f}; engine - plain: max {err.worst:.3e} rms {err.rms:.3e}; "
+          f"plain with bfloat16 activations - plain: max {noise.worst:.3e} rms {noise.rms:.3e}", flush=True)  # fmt: skip
+    if dtype == "float32":
+        assert err.worst <= 5e-5 * max(scale, 1.0)
+    else:
+        assert err.rms <= 1.25 * noise.rms and err.worst <= 2.0 * noise.worst
