@@ -86,29 +86,91 @@ def live_token_bound(steps, unit=64):
     return worst
 
 
-def run_and_compare(replay, steps, requests: dict, raw, weights, reference_cache: dict, plain_kwargs=None):
-    """Feed `steps` to a `Replay`; returns (largest |difference|, largest |reference|, rows compared).
-    plain_kwargs: how the plain model runs (default: float64 on the CPU, the loop form)."""
+class Spread:
+    """Largest and root-mean-square of the differences added to it."""
+
+    def __init__(self):
+        self.worst, self.sum_sq, self.count = 0.0, 0.0, 0
+
+    def add(self, diff):
+        self.worst = max(self.worst, float(diff.abs().max()))
+        self.sum_sq += float(diff.double().pow(2).sum())
+        self.count += diff.numel()
+
+    @property
+    def rms(self):
+        return (self.sum_sq / max(1, self.count)) ** 0.5
+
+
+class Comparison:
+    """What a trace's wanted rows are against the plain model: `err` engine - plain; `noise` the plain
+    model with its activations rounded to bfloat16 - plain (filled when asked for); `scale` the largest
+    |logit| of the plain model; `rows` compared.  Unpacks as (largest |difference|, scale, rows)."""
+
+    def __init__(self):
+        self.err, self.noise, self.scale, self.rows = Spread(), Spread(), 0.0, 0
+
+    def __iter__(self):
+        return iter((self.err.worst, self.scale, self.rows))
+
+
+# 32-bit: the engine and the float64 plain model differ by float32 rounding, a few 1e-6 of the largest logit.
+TOL_FLOAT32 = 2e-5
+# bfloat16: the engine may be as far from the exact logits as the plain model itself moves when its
+# activations are rounded to bfloat16 at the places where an engine that stores them so must round them
+# (tests/plain_qwen3.py `storage`), times these factors: root mean square over every compared logit, and
+# the largest single difference (the extreme of thousands of draws: it scatters more).  Over the 143
+# comparisons of tests/test_model_gpu.py the engine came to 1.09 and 1.33 of the plain model's own noise
+# at most; a fault of the cache or a kernel moves logits by their own size, tens of times the noise.
+BF16_RMS_FACTOR, BF16_WORST_FACTOR = 1.25, 2.0
+
+
+def within_bounds(result: Comparison, dtype: str, tol32: float = TOL_FLOAT32) -> None:
+    if dtype == "float32":
+        assert result.err.worst <= tol32 * max(result.scale, 1.0), \
+            f"float32: |difference| {result.err.worst:.3e} against |logits| {result.scale:.3e}"  # fmt: skip
+        return
+    assert result.noise.count == result.err.count and result.noise.count > 0, "the rounding noise was not measured"
+    assert result.err.rms <= BF16_RMS_FACTOR * result.noise.rms and result.err.worst <= BF16_WORST_FACTOR * result.noise.worst, (
+        f"bfloat16: engine - plain rms {result.err.rms:.3e} max {result.err.worst:.3e}; "
+        f"rounding alone moves the plain model by rms {result.noise.rms:.3e} max {result.noise.worst:.3e}")  # fmt: skip
+
+
+def plain_rows(raw, weights, ids, cache: dict, key, rounded: bool, plain_kwargs=None):
+    """The plain model's logits of a whole sequence (cached under `key`): exact, or with bfloat16 activations."""
+    key = (key, "rounded") if rounded else key
+    if key not in cache:
+        kwargs = dict(plain_kwargs or {})
+        if rounded:
+            kwargs.update(batched=True, storage=torch.bfloat16)
+        cache[key] = plain.logits(raw, weights, ids, **kwargs).float().cpu()
+    return cache[key]
+
+
+def run_and_compare(replay, steps, requests: dict, raw, weights, reference_cache: dict, plain_kwargs=None, noise=False):
+    """Feed `steps` to a `Replay` and compare every wanted row with the plain model's logits of the whole
+    sequence at that place; returns a `Comparison`.
+    plain_kwargs: how the plain model runs (default: float64 on the CPU, the loop form).
+    noise: also measure what rounding to bfloat16 alone does to the plain model at the same rows."""
     at = {rid: 0 for rid in requests}
-    worst, scale, rows = 0.0, 0.0, 0
+    result = Comparison()
     for s in steps:
         logits = replay.step(s["entries"], s["end"])
         k = 0
         for e in s["entries"]:
             rid = e["id"]
-            if rid not in reference_cache:
-                reference_cache[rid] = plain.logits(raw, weights, requests[rid], **(plain_kwargs or {})).float().cpu()
-            ref = reference_cache[rid]
+            ref = plain_rows(raw, weights, requests[rid], reference_cache, rid, False, plain_kwargs)
             for w in e["want"]:
-                got = logits[k]
                 want = ref[at[rid] + w]
-                worst = max(worst, float((got - want).abs().max()))
-                scale = max(scale, float(want.abs().max()))
+                result.err.add(logits[k] - want)
+                if noise:
+                    result.noise.add(plain_rows(raw, weights, requests[rid], reference_cache, rid, True, plain_kwargs)[at[rid] + w] - want)
+                result.scale = max(result.scale, float(want.abs().max()))
                 k += 1
-                rows += 1
+                result.rows += 1
             at[rid] += len(e["tokens"])
         assert (logits is None and k == 0) or logits.shape[0] == k
-    return worst, scale, rows
+    return result
 
 
 def random_ids(vocab, n, seed):

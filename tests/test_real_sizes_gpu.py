@@ -78,9 +78,9 @@ def test_every_layer_of_qwen3_8b_sizes_in_a_mixed_trace():
         del replay, model
         torch.cuda.empty_cache()
         rows = scale = 0
-        err = Spread()  # engine against the exact plain model
-        near = Spread()  # engine against the plain model with bfloat16 activations
-        noise = Spread()  # what bfloat16 activations alone do to the plain model
+        err = rc.Spread()  # engine against the exact plain model
+        near = rc.Spread()  # engine against the plain model with bfloat16 activations
+        noise = rc.Spread()  # what bfloat16 activations alone do to the plain model
         for rid, place, row in got:
             if rid not in exact_logits:
                 exact_logits[rid] = plain.logits(raw, exact, requests[rid], **PLAIN).float().cpu()
@@ -105,20 +105,6 @@ def test_every_layer_of_qwen3_8b_sizes_in_a_mixed_trace():
             # figure; the largest of 170 million differences: twice its like).
             assert err.rms <= 1.25 * noise.rms and err.worst <= 2.0 * noise.worst
             assert near.rms <= 1.5 * noise.rms
-
-
-class Spread:
-    def __init__(self):
-        self.worst, self.sum_sq, self.count = 0.0, 0.0, 0
-
-    def add(self, diff):
-        self.worst = max(self.worst, float(diff.abs().max()))
-        self.sum_sq += float(diff.double().pow(2).sum())
-        self.count += diff.numel()
-
-    @property
-    def rms(self):
-        return (self.sum_sq / max(1, self.count)) ** 0.5
 
 
 def wanted_rows(replay, steps):
@@ -235,7 +221,7 @@ def test_layer_sizes_of_every_model_the_benchmark_names(size, dtype, products):
         ops.fix_library_choices(was_fixed)
     assert replay.manager.num_free == replay.manager.num_blocks and len(got) == 65 + 66 + 3 + 2 * (64 + 32 + 16 + 12 + 8 + 3 + 1)
     assert sorted(n for n, _ in replay.runner.decode_graphs.graphs) == [1, 4, 8, 16, 32, 64]
-    err, noise, scale = Spread(), Spread(), 0.0
+    err, noise, scale = rc.Spread(), rc.Spread(), 0.0
     logits = {}
     for rid, place, row in got:
         if rid not in logits:
