@@ -62,6 +62,22 @@ class StateLayerView:
         self.state, self.row_slots, self.writes = state, row_slots, writes
 
 
+class RowSplit:
+    """A step's rows sorted as one kind of mixer asked (`Mixer.row_split` = (short, tile)):
+    short_tokens [Ns] int32: the tokens of rows with at most `short` tokens, those that see most keys first;
+    long_tiles [Nt, 4] int32: (first flat token, count, row, first position) per `tile` consecutive tokens
+    of longer rows, those that see most keys first; max_short_context: host bound on the context of a
+    short token."""
+
+    def __init__(self, short: int, tile: int):
+        if short < 0 or tile < 1:
+            raise ValueError(f"a row split is (short >= 0, tile >= 1), not {(short, tile)}")
+        self.short, self.tile = short, tile
+        self.tokens, self.tiles, self.max_short_context = [], [], 0
+        self.short_tokens = self.long_tiles = None  # on the device once the step is packed
+        self.num_short_tokens = self.num_long_tiles = 0
+
+
 class StepBatch:
     """The flat batch of one step, on the device.
 
@@ -69,29 +85,27 @@ class StepBatch:
     logits_rows [B'] int32                    flat indices of the wanted positions
     group_slots[g] [T], group_tables[g] [R, W_g] int32, per paged group
     all_tokens [T]: every token (in a decode step those with the longest contexts first);
-    with row_split = (short, tile), as the model's mixers ask (`Mixer.row_split`):
-    short_tokens [Ns]: tokens of rows with <= short tokens;
-    long_tiles [Nt, 4]: (first flat token, count, row, first position) per `tile` queries of longer rows
+    split((short, tile)): the rows sorted as a mixer asks (`RowSplit`), one for every distinct answer of
+    the model's mixers (`row_splits`), so that mixers with different kernels share a step;
     row_first, row_len, row_start, row_slots [R] int32 (for mixers with per-request state)
     """
 
     def __init__(self, rows, block_size: int, num_paged_groups: int, vocab_size: int, device, pools=None,
-                 staging=None, table_width: int = 0, max_context: int = 0, into=None, row_split=None):  # fmt: skip
+                 staging=None, table_width: int = 0, max_context: int = 0, into=None, row_splits=()):  # fmt: skip
         """table_width, max_context: lower bounds that make the layout of a step independent of
         its rows (a step whose kernels were captured in a graph is replayed with new contents).
-        into: an earlier batch of identical layout whose device buffer receives this one's arrays."""
+        into: an earlier batch of identical layout whose device buffer receives this one's arrays.
+        row_splits: the distinct (short, tile) that the model's mixers ask for."""
         if not rows:
             raise ValueError("a step needs at least one row")
         bs = block_size
-        short_row, tile_q = row_split if row_split is not None else (0, 0)
-        self.row_split = row_split
+        self.splits = {tuple(key): RowSplit(*key) for key in row_splits}
         tok, pos, trow, want = [], [], [], []
         slots = [[] for _ in range(num_paged_groups)]
-        short, tile_list = [], []
         row_first, row_len, row_start, row_slots = [], [], [], []
         widths = [max(1, table_width)] * num_paged_groups
         flat = 0
-        self.max_context = self.max_short_context = 0
+        self.max_context = 0
         for r, row in enumerate(rows):
             n, end = len(row.tokens), row.start + len(row.tokens)
             if n < 1 or row.start < 0:
@@ -126,14 +140,13 @@ class StepBatch:
             pos.extend(range(row.start, end))
             trow.extend([r] * n)
             want.extend(flat + w for w in row.want)
-            if row_split is None:
-                pass  # no mixer of this model wants its rows sorted
-            elif n <= short_row:
-                short.extend(range(flat, flat + n))
-                self.max_short_context = max(self.max_short_context, end)
-            else:
-                for q0 in range(0, n, tile_q):
-                    tile_list.append((flat + q0, min(tile_q, n - q0), r, row.start + q0))
+            for split in self.splits.values():
+                if n <= split.short:
+                    split.tokens.extend(range(flat, flat + n))
+                    split.max_short_context = max(split.max_short_context, end)
+                else:
+                    for q0 in range(0, n, split.tile):
+                        split.tiles.append((flat + q0, min(split.tile, n - q0), r, row.start + q0))
             self.max_context = max(self.max_context, end)
             row_first.append(flat)
             row_len.append(n)
@@ -143,11 +156,11 @@ class StepBatch:
 
         # Work items of the prefill kernel, the ones that see most keys first: the kernel hands
         # them out in this order and pairs the longest with the shortest on a compute unit.
-        tile_list.sort(key=lambda t: -(t[3] + t[1]))
-        short.sort(key=lambda t: -pos[t])  # single queries too: the longest contexts first
-        tiles = [v for t in tile_list for v in t]
+        for split in self.splits.values():
+            split.tiles.sort(key=lambda t: -(t[3] + t[1]))
+            split.tokens.sort(key=lambda t: -pos[t])  # single queries too: the longest contexts first
+            split.max_short_context = max(split.max_short_context, max_context if split.tokens else 0)
         self.max_context = max(self.max_context, max_context)
-        self.max_short_context = max(self.max_short_context, max_context if short else 0)
         T, R = flat, len(rows)
         tables = []
         for g in range(num_paged_groups):
@@ -164,9 +177,11 @@ class StepBatch:
         if T == R and T > 1:
             every = np.argsort(-np.asarray(pos, dtype=np.int64), kind="stable")
         fields = [("token_ids", tok), ("positions", pos), ("tok_row", trow), ("logits_rows", want),
-                  ("all_tokens", every), ("short_tokens", short), ("long_tiles", tiles),
-                  ("row_first", row_first), ("row_len", row_len), ("row_start", row_start),
+                  ("all_tokens", every), ("row_first", row_first), ("row_len", row_len), ("row_start", row_start),
                   ("row_slots", row_slots)]  # fmt: skip
+        for j, split in enumerate(self.splits.values()):
+            fields.append((f"short{j}", split.tokens))
+            fields.append((f"tiles{j}", [v for t in split.tiles for v in t]))
         for g in range(num_paged_groups):
             fields.append((f"slots{g}", slots[g]))
             fields.append((f"tables{g}", tables[g].reshape(-1)))
@@ -205,8 +220,9 @@ class StepBatch:
         self.token_ids, self.positions, self.tok_row = parts["token_ids"], parts["positions"], parts["tok_row"]
         self.logits_rows, self.num_logits = parts["logits_rows"], len(want)
         self.all_tokens = parts["all_tokens"]
-        self.short_tokens, self.num_short_tokens = parts["short_tokens"], len(short)
-        self.long_tiles, self.num_long_tiles = parts["long_tiles"].view(-1, 4), len(tiles) // 4
+        for j, split in enumerate(self.splits.values()):
+            split.short_tokens, split.num_short_tokens = parts[f"short{j}"], len(split.tokens)
+            split.long_tiles, split.num_long_tiles = parts[f"tiles{j}"].view(-1, 4), len(split.tiles)
         self.row_first, self.row_len = parts["row_first"], parts["row_len"]
         self.row_start, self.row_slots = parts["row_start"], parts["row_slots"]
         self.group_slots = [parts[f"slots{g}"] for g in range(num_paged_groups)]
@@ -216,6 +232,14 @@ class StepBatch:
         self.pools = pools
         self.shared = {}  # per-step results that parts share (rotary tables, ...)
 
+    def split(self, key) -> RowSplit:
+        """The rows sorted as a mixer whose `row_split()` is `key` needs them."""
+        found = self.splits.get(tuple(key))
+        if found is None:
+            raise ValueError(f"this step's rows are sorted for {sorted(self.splits)}, not for {tuple(key)}: "
+                             "the step is packed with every split that the model's mixers ask for")  # fmt: skip
+        return found
+
     def advance(self, rows) -> bool:
         """The next decode step of the same requests, in place: every row brings the one token
         that follows the row packed last, from the same block tables, so only the token, its
@@ -224,6 +248,8 @@ class StepBatch:
         old_rows, bs = self.host_rows, self.block_size
         if len(rows) != len(old_rows) or self.num_tokens != len(old_rows):
             return False
+        if any(split.num_long_tiles for split in self.splits.values()):
+            return False  # a split without single queries lists positions per tile, which this does not move on
         for new, old in zip(rows, old_rows):
             if (len(new.tokens) != 1 or new.tables is not old.tables or new.store != old.store or new.want != old.want
                     or new.state_slot != old.state_slot or new.start != old.start + (1 if new.store else 0)):
@@ -265,8 +291,11 @@ class StepBatch:
         return True
 
     def cache_view(self, cache_id: int, writes: bool):
-        """The view of cache `cache_id` for a mixer in this step."""
-        kind, gi, _ = self.pools.manager.group_of_cache[cache_id]
+        """The view of cache `cache_id` for a mixer in this step; None for a mixer that keeps nothing."""
+        found = self.pools.manager.group_of_cache.get(cache_id)
+        if found is None:
+            return None
+        kind, gi, _ = found
         if kind == "paged":
             _, k_pages, v_pages = self.pools.pages(cache_id)
             return PagedLayerView(k_pages, v_pages, self.group_slots[gi], self.group_tables[gi], writes, self.block_size)

@@ -62,6 +62,28 @@ class PhaseTimes:
         return {k: round(v / max(1, self.steps) * 1e6, 1) for k, v in self.seconds.items()}
 
 
+_capture_primer = None  # a trivial captured graph that lives as long as the process
+
+
+def _prime_capture(device) -> None:
+    """Once per process, before the first capture under inference mode: a trivial capture outside it,
+    kept alive.  torch keeps the random generator's state for captures in tensors that it makes when
+    the first graph of the process registers (and drops when the last one is destroyed) and fills in
+    place at every capture; made under inference mode they would refuse that update in a later capture
+    outside it (a caller's own graphs, after this engine's).  While this graph lives they stay as they
+    were made here."""
+    global _capture_primer
+    if _capture_primer is not None:
+        return
+    with torch.inference_mode(False):
+        scratch = torch.zeros(1, device=device)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            scratch += 1
+    _capture_primer = (graph, scratch)
+
+
 def _bucket(n: int, steps) -> int:
     for s in steps:
         if n <= s:
@@ -177,6 +199,7 @@ class DecodeGraphs:
         torch.cuda.synchronize()
         ops.settle_library_choices()  # what the warm-up tried among the library's products is decided now
         batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
+        _prime_capture(r.device)
         graph = torch.cuda.CUDAGraph()
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
@@ -258,7 +281,7 @@ class ModelRunner:
         self.sampler = Sampler(self.device)
         self.staging = Staging(self.device)
         self.vocab_size = model.plan.vocab_size
-        self.row_split = model.row_split()  # how the model's mixers want the rows of a step sorted
+        self.row_splits = model.row_splits()  # how the model's mixers want the rows of a step sorted
         self.decode_graphs = DecodeGraphs(self) if use_graphs else None
         self._token_buffers = []  # pinned, used in turn: the sampled tokens of the steps on their way
         self._token_turn = 0
@@ -266,7 +289,7 @@ class ModelRunner:
 
     def prepare(self, rows, **layout) -> StepBatch:
         return StepBatch(rows, self.manager.block_size, len(self.manager.paged_groups), self.vocab_size,
-                         self.device, pools=self.pools, staging=self.staging, row_split=self.row_split,
+                         self.device, pools=self.pools, staging=self.staging, row_splits=self.row_splits,
                          **layout)  # fmt: skip
 
     @torch.inference_mode()

@@ -77,11 +77,6 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.running) or bool(self.waiting)
 
-    @property
-    def allocator(self):
-        """The page allocator of the first paged group (the only one of a model with one kind of cache)."""
-        return self.manager.paged_groups[0].allocator
-
     def add(self, seq: Sequence) -> None:
         seq.cache = self.manager.new_request()
         self.waiting.append(seq)

@@ -75,11 +75,6 @@ class Sequence:
         """A copy of the generated tokens; `num_output_tokens` counts them without one."""
         return self.token_ids[self.num_prompt_tokens :]
 
-    @property
-    def block_table(self) -> list:
-        """The first paged group's table (the only one, for a model with one kind of cache)."""
-        return self.cache.tables[0] if self.cache.tables else []
-
     def reaches_end(self, num_new_tokens: int) -> bool:
         """Whether computing `num_new_tokens` more covers every known token: only then is
         there a next token to predict (reference atomserve/sequence.py:93-100)."""

@@ -81,13 +81,11 @@ class DecoderModel:
         return requests
 
     # ---- one pass ---------------------------------------------------------------------
-    def row_split(self):
-        """How the mixers want the rows of a step sorted for their kernels (`Mixer.row_split`): one
-        answer for the whole model, or None if no mixer cares."""
-        wanted = {split for block in self.blocks for split in [block.parts()["mixer"].row_split()] if split is not None}
-        if len(wanted) > 1:
-            raise ValueError(f"the mixers of this model want their rows split in different ways: {sorted(wanted)}")
-        return next(iter(wanted), None)
+    def row_splits(self) -> tuple:
+        """How the mixers want the rows of a step sorted for their kernels: every distinct answer of
+        `Mixer.row_split` among the layers (none if no mixer cares); a step is packed once for each."""
+        return tuple(sorted({split for block in self.blocks for split in [block.parts()["mixer"].row_split()]
+                             if split is not None}))  # fmt: skip
 
     def forward(self, step, logits: torch.Tensor = None) -> torch.Tensor:
         """Run this step's tokens through every run of the plan; returns fp32 logits

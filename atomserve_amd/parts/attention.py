@@ -40,7 +40,19 @@ class Attention(Mixer):
                 f"head_dim {s.head_dim} is not supported by the attention kernels "
                 f"(a multiple of {chunk}, at most {ops.SINGLE_QUERY_MAX_HEAD_DIM})"
             )
+        # What the kernels compute and nothing else: a per-head RMSNorm, and a rotation of the pairs
+        # (i, i + R/2) of a head's first R coordinates by angles that the position part tabulates.
+        if s.qk_norm is not None and s.qk_norm.kind != "rmsnorm":
+            raise ValueError(f"the attention kernels norm heads by 'rmsnorm' only, not by {s.qk_norm.kind!r}")
+        if s.qk_norm is not None and s.qk_norm.size != s.head_dim:
+            raise ValueError(f"the per-head norm has {s.qk_norm.size} gains, a head {s.head_dim} coordinates")
         self.position = build("position", s.position, env) if s.position is not None else None
+        if self.position is not None and getattr(self.position, "pairs", None) != "half":
+            raise ValueError(
+                f"the attention kernels rotate the pairs (i, i + R/2) by a table of cosines and sines "
+                f"(a position part that declares pairs = 'half'); {s.position.kind!r} declares "
+                f"{getattr(self.position, 'pairs', None)!r}"
+            )
         self.q_norm_weight = self.k_norm_weight = None
 
     def weight_decls(self) -> dict:
@@ -123,13 +135,12 @@ class Attention(Mixer):
             ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
                                   cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
             return
-        if step.row_split != self.row_split():
-            raise ValueError(f"this step's rows are sorted as {step.row_split}, the attention kernels need {self.row_split()}")
-        if step.num_short_tokens:
-            ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.short_tokens, step.positions, step.tok_row,
-                                  cache.block_tables, out, s.scale, s.window, step.max_short_context)  # fmt: skip
-        if step.num_long_tiles:
-            ops.attn_prefill(q, cache.k_pages, cache.v_pages, step.long_tiles, cache.block_tables, out, s.scale,
+        rows = step.split(self.row_split())
+        if rows.num_short_tokens:
+            ops.attn_single_query(q, cache.k_pages, cache.v_pages, rows.short_tokens, step.positions, step.tok_row,
+                                  cache.block_tables, out, s.scale, s.window, rows.max_short_context)  # fmt: skip
+        if rows.num_long_tiles:
+            ops.attn_prefill(q, cache.k_pages, cache.v_pages, rows.long_tiles, cache.block_tables, out, s.scale,
                              s.window, step.max_context)  # fmt: skip
 
 

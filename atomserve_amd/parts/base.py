@@ -164,6 +164,12 @@ class Norm(Part):
 
 
 class Position(Part):
+    # How a mixer is to apply what `prepare` returns.  "half": an fp32 table [T, R/2, 2] of (cos, sin) by which
+    # the pairs (i, i + R/2) of a head's first R coordinates turn (scaled, partial or slowed rotations are
+    # other tables of the same kind).  A part of another layout (neighbouring pairs, something added to the
+    # scores) names it here, and a mixer whose kernels do not compute that layout refuses the part.
+    pairs: Optional[str] = None
+
     def prepare(self, step: Any) -> Any:
         raise NotImplementedError
 

@@ -15,6 +15,7 @@ from atomserve_amd.parts.base import Position, register
 
 class RotaryHalf(Position):
     capturable = True
+    pairs = "half"
 
     def __init__(self, spec, env):
         super().__init__(spec, env)

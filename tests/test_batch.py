@@ -8,10 +8,11 @@ from atomserve_amd.cache.manager import RELEASED
 from atomserve_amd.engine.batch import Row, StepBatch
 
 BS = 4
+ATTENTION = (8, 64)  # rows of up to 8 tokens as single queries, longer ones in tiles of 64
 
 
 def pack(rows, **layout):
-    return StepBatch(rows, BS, 2, 100, "cpu", **{"row_split": (8, 64), **layout})
+    return StepBatch(rows, BS, 2, 100, "cpu", **{"row_splits": [ATTENTION], **layout})
 
 
 def decode_rows(tables, starts, tokens, filler):
@@ -27,10 +28,10 @@ def test_rows_are_flattened_with_slots_tables_and_tiles():
     assert b.group_slots[0].tolist() == [2 * BS + 0, 2 * BS + 1, 2 * BS + 2, 3 * BS + 2]
     assert b.group_slots[1].tolist() == [1 * BS + 0, 1 * BS + 1, 1 * BS + 2, 4 * BS + 2]
     assert b.group_tables[0].tolist() == [[5, 2], [3, 0]]
-    assert b.short_tokens.tolist() == [2, 1, 0, 3] and b.num_long_tiles == 0  # those that see most keys first
+    assert b.split(ATTENTION).short_tokens.tolist() == [2, 1, 0, 3] and b.split(ATTENTION).num_long_tiles == 0  # those that see most keys first
     long = pack([Row(list(range(70)), 0, [list(range(20)), list(range(20))], []), Row([1] * 9, 64, [list(range(20, 40))] * 2, [])])
     # work items of the prefill kernel, the one that sees most keys first
-    assert long.long_tiles.tolist() == [[70, 9, 1, 64], [64, 6, 0, 64], [0, 64, 0, 0]]
+    assert long.split(ATTENTION).long_tiles.tolist() == [[70, 9, 1, 64], [64, 6, 0, 64], [0, 64, 0, 0]]
     # a prompt's slots are computed as arrays: the same places as token by token, from the middle of a page on
     table = [(7 * i + 3) % 31 for i in range(30)]  # 30 different pages, in no order
     start = BS + 3
@@ -89,14 +90,30 @@ def test_a_decode_step_lists_its_tokens_longest_context_first():
 
 def test_rows_are_sorted_only_for_mixers_that_ask():
     """Short rows and tiles are what the attention kernels of this package want; a model whose
-    mixers ask for nothing gets its rows as they come, another split gives other lists."""
+    mixers ask for nothing gets its rows as they come, another split gives other lists, and mixers
+    that ask for different splits each find theirs in the same step."""
     rows = [Row([1, 2, 3], 0, [[2], [1]], [2]), Row(list(range(10)), 0, [[3, 0, 6], [4, 5, 7]], [9])]
     plain = StepBatch(rows, BS, 2, 100, "cpu")
-    assert plain.num_short_tokens == 0 and plain.num_long_tiles == 0
-    assert plain.row_first.tolist() == [0, 3] and plain.row_len.tolist() == [3, 10]
-    split = StepBatch(rows, BS, 2, 100, "cpu", row_split=(2, 4))
-    assert split.num_short_tokens == 0
-    assert sorted(split.long_tiles.tolist()) == [[0, 3, 0, 0], [3, 4, 1, 0], [7, 4, 1, 4], [11, 2, 1, 8]]
+    assert plain.splits == {} and plain.row_first.tolist() == [0, 3] and plain.row_len.tolist() == [3, 10]
+    with pytest.raises(ValueError, match="sorted for"):
+        plain.split(ATTENTION)
+    both = StepBatch(rows, BS, 2, 100, "cpu", row_splits=[(2, 4), ATTENTION, (3, 8)])
+    fine = both.split((2, 4))
+    assert fine.num_short_tokens == 0 and fine.max_short_context == 0
+    assert sorted(fine.long_tiles.tolist()) == [[0, 3, 0, 0], [3, 4, 1, 0], [7, 4, 1, 4], [11, 2, 1, 8]]
+    coarse = both.split(ATTENTION)
+    assert coarse.short_tokens.tolist() == [2, 1, 0] and coarse.long_tiles.tolist() == [[3, 10, 1, 0]] and coarse.max_short_context == 3
+    third = both.split((3, 8))
+    assert third.short_tokens.tolist() == [2, 1, 0] and sorted(third.long_tiles.tolist()) == [[3, 8, 1, 0], [11, 2, 1, 8]]
+    alone = StepBatch(rows, BS, 2, 100, "cpu", row_splits=[(3, 8)]).split((3, 8))
+    assert alone.long_tiles.tolist() == third.long_tiles.tolist()  # a split does not depend on its neighbours
+    with pytest.raises(ValueError):
+        StepBatch(rows, BS, 2, 100, "cpu", row_splits=[(2, 0)])
+    # a split without single queries lists positions per tile: such a decode step is packed anew, not moved on
+    tables = [[[5, 2], [7, 1]], [[3], [4]]]
+    tiled = StepBatch([Row([1], 6, tables[0], [0]), Row([2], 2, tables[1], [0])], BS, 2, 100, "cpu", row_splits=[(0, 4)])
+    assert tiled.split((0, 4)).num_long_tiles == 2
+    assert not tiled.advance([Row([3], 7, tables[0], [0]), Row([4], 3, tables[1], [0])])
 
 
 def test_pages_given_back_by_a_window_leave_the_captured_table():

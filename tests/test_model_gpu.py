@@ -687,3 +687,27 @@ def test_warm_up_captures_the_decode_steps_ahead(setup):
     got = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
     assert got == [plain.greedy(raw, weights, p, 6) for p in prompts]
     assert len(graphs) == 4 and engine.stats()["kv_blocks_used"] == 0
+
+
+def test_a_callers_own_graph_after_the_engines(setup):
+    """The engine captures its decode steps under inference mode; a capture that the same process makes
+    afterwards outside inference mode (torch fills the random generator's capture state in place, in
+    tensors made at the process's first capture) goes through and replays."""
+    from atomserve_amd.config import EngineConfig
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.weights import load_model
+
+    name, raw, weights, path, _ = setup
+    model, _, _ = load_model(path, torch.float32, "cuda:0")
+    engine = create_engine(model, EngineConfig(block_size=16, num_blocks=16, max_model_len=64, max_num_seqs=2))
+    assert engine.warm_up() == 2
+    assert not torch.is_inference_mode_enabled()
+    x = torch.zeros(8, device="cuda:0")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        x += 1
+    graph.replay()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert x.tolist() == [2.0] * 8

@@ -382,6 +382,8 @@ def make_slowed_rotary():
         """Rotation of half of each head, by angles of position / slowdown: the table the attention
         part hands to its kernel, computed here with library calls."""
 
+        pairs = "half"  # a table of (cos, sin) for the pairs (i, i + R/2), as the attention kernels rotate
+
         def prepare(self, step):
             s = self.spec
             key = ("toy_slowed", s.rotary_dim, s.theta, s.slowdown)
@@ -636,7 +638,7 @@ def test_attention_part_alone(dtype):
     outs, at = [], 0
     for n in (20, 1, 1, 8):
         manager.reserve(rc, at, n)
-        batch = StepBatch([Row([0] * n, at, rc.tables, [])], 16, 1, 10, DEV, pools=pools, row_split=mixer.row_split())
+        batch = StepBatch([Row([0] * n, at, rc.tables, [])], 16, 1, 10, DEV, pools=pools, row_splits=[mixer.row_split()])
         outs.append(mixer.forward(x[at : at + n].to(DEV).to(dtype), batch, batch.cache_view(0, True)).float().cpu())
         at += n
     tol = (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, float(ref.abs().max()))
@@ -735,3 +737,127 @@ def test_a_plan_scales_its_embeddings_and_caps_its_logits(dtype, device=DEV):
     # the cap's slope is at most one: an error of the scaled logits passes through no larger
     assert (got - ref).abs().max() <= tol * max(1.0, float(uncapped.abs().max()))
     assert 0.7 * cap < ref.abs().max() < cap  # the cap bites
+
+
+# ---- two mixers that want a step's rows sorted in different ways ---------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class PositionGateSpec:
+    kind: str
+    hidden_size: int
+    period: float
+
+
+def make_position_gate_mixer():
+    from atomserve_amd.parts.base import Mixer, WeightDecl
+
+    class PositionGate(Mixer):
+        """y_t = gain * h_t * cos(position_t / period).  It keeps nothing; it asks for every row in work
+        items of up to four consecutive tokens, single tokens included, and takes each token's position
+        from its work item: another sorting of the step's rows than the attention part asks for."""
+
+        SPLIT = (0, 4)
+
+        def weight_decls(self):
+            return {"gain": WeightDecl((self.spec.hidden_size,), role="vector")}
+
+        def row_split(self):
+            return self.SPLIT
+
+        def forward(self, h, step, cache):
+            out = torch.full_like(h, float("nan"))
+            items = step.split(self.SPLIT)
+            assert items.num_short_tokens == 0
+            for first, count, row, position in items.long_tiles.cpu().tolist():
+                assert 1 <= count <= 4 and step.host_rows[row].start <= position
+                at = torch.arange(position, position + count, device=h.device, dtype=torch.float32)
+                gate = torch.cos(at / self.spec.period)[:, None]
+                out[first : first + count] = (h[first : first + count].float() * self.gain.float() * gate).to(h.dtype)
+            return out
+
+    return PositionGate
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mixers_that_sort_the_rows_differently_share_a_step(dtype):
+    """Odd layers gate the stream by position through work items of four tokens, even layers attend:
+    the step is packed once for each of the two sortings, and each mixer finds its own."""
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+    from atomserve_amd.parts.attention import SHORT_ROW, TILE_Q
+    from atomserve_amd.parts.base import register
+
+    register("mixer", "toy_position_gate", make_position_gate_mixer(), replace=True)
+    qwen = architecture_for(TINY_A)
+    period = 7.0
+
+    def build_plan(c):
+        plan = qwen.build_plan(c)
+        layers = tuple(dataclasses.replace(layer, mixer=PositionGateSpec("toy_position_gate", c.hidden_size, period)) if i % 2 else layer
+                       for i, layer in enumerate(plan.layers))  # fmt: skip
+        return dataclasses.replace(plan, layers=layers)
+
+    def checkpoint_map(c):
+        names = {k: v for k, v in qwen.checkpoint_map(c).items()
+                 if not any(k.startswith(f"layers.{i}.mixer.") for i in range(1, c.num_layers, 2))}  # fmt: skip
+        for i in range(1, c.num_layers, 2):
+            names[f"layers.{i}.mixer.gain"] = [f"model.layers.{i}.gate.gain"]
+        return names
+
+    def checkpoint_shapes(c):
+        shapes = {k: v for k, v in qwen.checkpoint_shapes(c).items()
+                  if not any(k.startswith(f"model.layers.{i}.self_attn.") for i in range(1, c.num_layers, 2))}  # fmt: skip
+        for i in range(1, c.num_layers, 2):
+            shapes[f"model.layers.{i}.gate.gain"] = ((c.hidden_size,), "vector")
+        return shapes
+
+    arch = register_architecture(
+        Architecture("GatedByPositionForCausalLM", qwen.parse_config, build_plan, checkpoint_map, checkpoint_shapes), replace=True
+    )
+    raw = {**TINY_A, "architectures": ["GatedByPositionForCausalLM"], "num_hidden_layers": 4}
+    w = plain_random_weights(raw, seed=12, std=0.2, gain_std=0.2)
+    for i in (1, 3):
+        for k in [k for k in w if k.startswith(f"model.layers.{i}.self_attn.")]:
+            del w[k]
+        w[f"model.layers.{i}.gate.gain"] = (1 + 0.2 * torch.randn(raw["hidden_size"])).bfloat16().float()
+    engine = build_engine(arch, raw, w, dtype)
+    assert engine.runner.row_splits == ((0, 4), (SHORT_ROW, TILE_Q))
+
+    def reference(ids):
+        cfg = plain.normalise_config(raw)
+        wd = {k: v.double() for k, v in w.items()}
+        pos = torch.arange(len(ids))
+        x = plain.embed(wd["model.embed_tokens.weight"], torch.as_tensor(ids))
+        for i in range(4):
+            p = f"model.layers.{i}."
+            h = plain.rms_norm(x, wd[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+            if i % 2:
+                x = x + h * wd[p + "gate.gain"] * torch.cos(pos.double() / period)[:, None]
+            else:
+                x = x + plain.attention_layer(h, wd, p, cfg, pos)
+            h = plain.rms_norm(x, wd[p + "post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+            x = x + plain.swiglu(h, wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"], wd[p + "mlp.down_proj.weight"])
+        x = plain.rms_norm(x, wd["model.norm.weight"], cfg["rms_norm_eps"])
+        return (x @ wd["model.embed_tokens.weight"].T).float()
+
+    a = torch.randint(0, 256, (90,), generator=torch.Generator().manual_seed(21)).tolist()
+    b = torch.randint(0, 256, (31,), generator=torch.Generator().manual_seed(22)).tolist()
+    ref = {"a": reference(a), "b": reference(b)}
+    caches, got = {}, {"a": [], "b": []}
+    # a prompt of 70 tokens (tiles of 64 for one mixer, of 4 for the other) beside a short row, then
+    # single tokens beside a portion, then decode steps of both
+    logits = step_rows(engine, caches, [("a", a[:70], list(range(70))), ("b", b[:3], [0, 1, 2])])
+    got["a"].append(logits[:70]); got["b"].append(logits[70:])  # noqa: E702
+    logits = step_rows(engine, caches, [("b", b[3:4], [0]), ("a", a[70:83], list(range(13)))])
+    got["b"].append(logits[:1]); got["a"].append(logits[1:])  # noqa: E702
+    logits = step_rows(engine, caches, [("b", b[4:24], list(range(20)))])
+    got["b"].append(logits)
+    for i in range(7):
+        logits = step_rows(engine, caches, [("a", [a[83 + i]], [0]), ("b", [b[24 + i]], [0])])
+        got["a"].append(logits[:1]); got["b"].append(logits[1:])  # noqa: E702
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    for name in "ab":
+        assert (torch.cat(got[name]) - ref[name]).abs().max() <= tol * max(1.0, ref[name].abs().max()), name
+    for rc, _ in caches.values():
+        engine.scheduler.manager.release(rc)
+    assert engine.scheduler.manager.num_free == engine.scheduler.manager.num_blocks

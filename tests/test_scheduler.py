@@ -14,6 +14,12 @@ from atomserve_amd.engine.scheduler import Scheduler
 from atomserve_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus, StepResult
 
 EOS = 999
+
+
+def table_of(seq) -> list:
+    """The request's block table in the one group of pages these schedulers have."""
+    return seq.cache.tables[0] if seq.cache.tables else []
+
 GREEDY = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
 
 
@@ -25,12 +31,12 @@ class FakeRunner:
         results = []
         for seq, n in zip(out.seqs, out.num_new_tokens, strict=True):
             start, end = seq.num_computed_tokens, seq.num_computed_tokens + n
-            assert end <= len(seq.block_table) * self.bs, "block table too small"
+            assert end <= len(table_of(seq)) * self.bs, "block table too small"
             for p in range(start, end):
-                self.slots[slot_of(seq.block_table, p, self.bs)] = seq.token_ids[p]
+                self.slots[slot_of(table_of(seq), p, self.bs)] = seq.token_ids[p]
             tokens = []
             if seq.reaches_end(n):
-                context = [self.slots[slot_of(seq.block_table, p, self.bs)] for p in range(end)]
+                context = [self.slots[slot_of(table_of(seq), p, self.bs)] for p in range(end)]
                 tokens.append(sum((i + 1) * t for i, t in enumerate(context)) % 500)
             results.append(StepResult(tokens, end))
         return results
@@ -44,7 +50,7 @@ def make(**config):
 def sharing_is_safe(s):
     bs, owners = s.config.block_size, {}
     for seq in s.running:
-        for i, page in enumerate(seq.block_table):
+        for i, page in enumerate(table_of(seq)):
             owners.setdefault(page, []).append((seq, i))
     for sharers in owners.values():
         if len(sharers) > 1:
@@ -110,7 +116,7 @@ def test_preemption_evicts_the_newest_and_requeues_it_first():
     out = s.schedule()  # both need a second page; only one can grow
     assert out.preempted == [new] and out.seqs == [old]
     assert s.waiting[0] is new and new.status is SequenceStatus.WAITING
-    assert new.num_computed_tokens == 0 and new.block_table == []
+    assert new.num_computed_tokens == 0 and table_of(new) == []
     # nobody is admitted in a step that had to preempt
     assert len(s.running) == 1
 
@@ -178,7 +184,7 @@ def test_abort_frees_running_and_waiting_requests():
     s.add(running)
     s.add(waiting)
     s.schedule()
-    assert running.status is SequenceStatus.RUNNING and running.block_table
+    assert running.status is SequenceStatus.RUNNING and table_of(running)
     assert s.abort(0) is running and s.abort(1) is waiting and s.abort(1) is None
     assert running.finish_reason == waiting.finish_reason == "abort"
     assert not s.has_work and s.manager.num_free == 16
@@ -227,7 +233,7 @@ def test_running_requests_share_a_prefix_and_pressure_keeps_outputs():
         s.update(out, runner.execute(out))
     s.add(b)
     out = s.schedule()
-    assert b.block_table[:3] == a.block_table[:3] and out.num_new_tokens == [1, 1]
+    assert table_of(b)[:3] == table_of(a)[:3] and out.num_new_tokens == [1, 1]
     s.update(out, runner.execute(out))
     drive(s, runner)
     assert a.output_ids == alone(system + [1, 2]) and b.output_ids == alone(system + [3])
