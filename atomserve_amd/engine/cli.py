@@ -102,6 +102,9 @@ def build_parser() -> argparse.ArgumentParser:
                    help="always take the library's first candidate for its matrix products instead of timing them at "
                         "start-up: bfloat16 results are then the same from run to run (a little slower at 17 to 64 "
                         "requests and for prompts)")  # fmt: skip
+    p.add_argument("--no-stream-copies", action="store_true",
+                   help="do not keep the weights a second time in the order the decode kernels read them: saves "
+                        "their bytes again (15 GB at Qwen3-8B sizes), decode steps are some 7 per cent slower")  # fmt: skip
     p.add_argument("--version", action="version", version=f"%(prog)s {__version__}")
     return p
 
@@ -119,14 +122,17 @@ def engine_config_for(args, bytes_per_block: int, max_positions: int):
     limit = min(max_positions, num_blocks * args.block_size)
     if args.max_model_len is not None:
         limit = min(limit, args.max_model_len)
-    return EngineConfig(
-        block_size=args.block_size,
-        num_blocks=num_blocks,
-        max_num_seqs=args.max_num_seqs,
-        max_num_batched_tokens=args.max_batched_tokens,
-        max_model_len=limit,
-        enable_prefix_caching=not args.no_prefix_caching,
-    )
+    try:
+        return EngineConfig(
+            block_size=args.block_size,
+            num_blocks=num_blocks,
+            max_num_seqs=args.max_num_seqs,
+            max_num_batched_tokens=args.max_batched_tokens,
+            max_model_len=limit,
+            enable_prefix_caching=not args.no_prefix_caching,
+        )
+    except ValueError as error:  # limits that contradict each other: a message, not a traceback
+        raise SystemExit(f"atomserve: {error}") from None
 
 
 def parse_ids(text: str) -> list:
@@ -172,7 +178,7 @@ def main(argv=None) -> int:
     config = arch.parse_config(raw)
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     print(f"Loading {args.model} ({args.dtype}, {arch.name}) ...", file=sys.stderr, flush=True)
-    model = DecoderModel(arch.build_plan(config), dtype, "cuda:0")
+    model = DecoderModel(arch.build_plan(config), dtype, "cuda:0", stream_copies=not args.no_stream_copies)
     if args.random_weights is not None:
         source = DictSource(random_checkpoint(arch, config, args.random_weights, dtype=dtype, device="cuda:0"))
         bind_checkpoint(model, arch, config, source, where="(random)")
@@ -188,9 +194,7 @@ def main(argv=None) -> int:
     if args.kv_mem_gb * 2**30 // block_bytes > 2**31 // args.block_size:  # slots are 32-bit integers
         args.kv_mem_gb = (2**31 // args.block_size) * block_bytes / 2**30
     engine_config = engine_config_for(args, block_bytes, model.plan.max_positions)
-    from atomserve_amd.kernels import ops
-
-    ops.fix_library_choices(args.fixed_products)
+    model.env.products.fix(args.fixed_products)
     engine = create_engine(model, engine_config, eos_ids(model_dir), seed=args.seed)
     engine.generate([[0]], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))  # compile and warm up
     engine.warm_up()  # and capture the decode steps of every batch size now, not at their first use
@@ -201,9 +205,12 @@ def main(argv=None) -> int:
         file=sys.stderr, flush=True,
     )  # fmt: skip
 
-    params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
-                            presence_penalty=args.presence_penalty, max_tokens=args.max_tokens, seed=args.seed,
-                            ignore_eos=args.ignore_eos)  # fmt: skip
+    try:
+        params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
+                                presence_penalty=args.presence_penalty, max_tokens=args.max_tokens, seed=args.seed,
+                                ignore_eos=args.ignore_eos).validated()  # fmt: skip
+    except ValueError as error:
+        raise SystemExit(f"atomserve: {error}") from None
     prompts = [parse_ids(p) for p in args.prompt_ids]
     if args.prompt_file:
         with open(args.prompt_file) as f:

@@ -34,7 +34,6 @@ from atomserve_amd.config.engine_config import EngineConfig
 from atomserve_amd.engine.runner import ModelRunner
 from atomserve_amd.engine.scheduler import Scheduler, StepPlan
 from atomserve_amd.engine.sequence import SamplingParams, Sequence, SequenceStatus
-from atomserve_amd.kernels import ops
 
 _END = object()  # last item of a request's stream
 
@@ -142,8 +141,7 @@ class Engine:
         longest = self.scheduler.config.max_model_len
         if not ids or len(ids) >= longest:
             raise ValueError(f"prompt has {len(ids)} tokens; must be 1 to {longest - 1}")
-        if params.max_tokens < 1:
-            raise ValueError("max_tokens must be at least 1")
+        params.validated()
         vocab = getattr(self.runner, "vocab_size", None)
         if vocab is not None and (min(ids) < 0 or max(ids) >= vocab):
             raise ValueError(f"prompt holds a token id outside the vocabulary of {vocab}")
@@ -218,6 +216,10 @@ class Engine:
         held = getattr(self.runner, "graph_bytes", None)
         if held is not None:
             report["graph_bytes"] = held()
+        model = getattr(self.runner, "model", None)
+        if model is not None:  # the weights, and their second copies in the order the decode kernels read them
+            report["weight_bytes"] = model.num_weight_bytes
+            report["stream_copy_bytes"] = model.num_stream_copy_bytes
         return report
 
     @property
@@ -346,5 +348,5 @@ def create_engine(model, engine_config: EngineConfig, eos_token_ids=frozenset(),
                            engine_config.max_num_seqs)  # fmt: skip
     runner = ModelRunner(model, manager)
     if runner.device.type == "cuda":
-        ops.tune_library_rows(engine_config.max_num_batched_tokens)  # what a step with a prompt's portion brings
+        model.env.products.tune_rows(engine_config.max_num_batched_tokens)  # what a step with a prompt's portion brings
     return Engine(runner, Scheduler(engine_config, eos_token_ids, manager), seed=seed)

@@ -56,7 +56,6 @@ class Replay:
 
         from atomserve_amd.cache.manager import CacheManager
         from atomserve_amd.engine.runner import ModelRunner
-        from atomserve_amd.kernels import ops
         from atomserve_amd.weights.loader import load_model
 
         self.log = log or (lambda msg: None)
@@ -74,7 +73,7 @@ class Replay:
         else:
             self.log(f"loading {model_dir} ({DTYPES[dtype]}) ...")
             self.model, self.arch, self.config = load_model(model_dir, torch_dtype, device)
-        ops.fix_library_choices(fixed_products)
+        self.model.env.products.fix(fixed_products)  # this model's products only: another engine of the process keeps its own
         self.block_size, self.max_live = block_size, max_live
         self.manager = CacheManager(self.model.cache_requests(), block_size, num_pages, max_live)
         self.runner = ModelRunner(self.model, self.manager)
@@ -83,10 +82,14 @@ class Replay:
 
     def step(self, entries: list, end: list):
         """Run one step; returns the logits of its wanted places as a CPU tensor, or None.
-        A step that cannot run (no room, too many requests) raises and changes nothing."""
+        A step that cannot run (a token outside the vocabulary, a wanted place outside its row, no room,
+        too many requests) raises before anything is taken and changes nothing.  If the pass itself
+        fails on the GPU, the requests that this step started are dropped with their pages, and the
+        pages it added to older requests stay theirs (they are given back when those requests end)."""
         from atomserve_amd.engine.batch import Row
 
         work, seen = [], set()
+        vocab = self.runner.vocab_size
         for e in entries:
             rid, tokens, want = e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]
             if rid in seen:
@@ -96,6 +99,11 @@ class Replay:
                 if want:
                     raise ValueError(f"request {rid!r} wants logits of a step in which it has no tokens")
                 continue
+            outside = [t for t in tokens if not 0 <= t < vocab]
+            if outside:
+                raise ValueError(f"request {rid!r}: token id {outside[0]} is outside the vocabulary of {vocab}")
+            if any(not 0 <= w < len(tokens) for w in want):
+                raise ValueError(f"request {rid!r} wants logits at places {want} outside its {len(tokens)} tokens")
             work.append((rid, tokens, want))
         fresh = [rid for rid, _, _ in work if rid not in self.live]
         if len(self.live) + len(fresh) > self.max_live:
@@ -113,7 +121,12 @@ class Replay:
                 for rid, tokens, want in work]  # fmt: skip
         logits = None
         if rows:
-            out = self.runner.step(rows)
+            try:
+                out = self.runner.step(rows)
+            except BaseException:
+                for rid in started:
+                    self.manager.release(self.live.pop(rid)[0])
+                raise
             if out.shape[0]:
                 logits = out.cpu()
             for rid, tokens, _ in work:

@@ -186,18 +186,19 @@ class DecodeGraphs:
             self.logits = torch.empty((self.most_rows, r.vocab_size), dtype=torch.float32, device=r.device)
         batch = r.prepare([self.filler() for _ in range(n)], table_width=width, max_context=context)
         out = self.logits[:n]
-        ops.tune_library_rows(n)  # a bucket's products come again at every replay: worth trying the library's candidates
+        products = r.model.env.products
+        products.tune_rows(n)  # a bucket's products come again at every replay: worth trying the library's candidates
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             r.model.forward(batch, logits=out)  # loads every library and warms the allocator before capture
             for _ in range(3):  # and while the library's products are still being tried, again
-                if not ops.library_trials_pending():
+                if not products.trials_pending():
                     break
                 r.model.forward(batch, logits=out)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        ops.settle_library_choices()  # what the warm-up tried among the library's products is decided now
+        products.settle()  # what the warm-up tried among the library's products is decided now
         batch.shared.clear()  # what parts computed once for the warm-up must be computed in the graph too
         _prime_capture(r.device)
         graph = torch.cuda.CUDAGraph()
@@ -329,7 +330,8 @@ class ModelRunner:
         """Runs a prompt that stores nothing at each of a few lengths (128, 192, 256, 384, ... up to `most_tokens`)
         until the library's candidates for its products have been tried and the fastest chosen; prompts
         of other lengths then take what the next length above them chose.  Returns the lengths run."""
-        if self.device.type != "cuda" or ops.library_choices_fixed():
+        products = self.model.env.products
+        if self.device.type != "cuda" or products.fixed:
             return []
         bs, lengths, n = self.manager.block_size, [], 128
         while n <= most_tokens:
@@ -337,14 +339,14 @@ class ModelRunner:
             n *= 2
         slot = self.pools.scrap_slot if self.manager.state_groups else -1
         for n in lengths:
-            ops.tune_library_rows(n)
+            products.tune_rows(n)
             tables = [[0] * -(-n // bs) for _ in self.manager.paged_groups]
             rows = [Row([0] * n, 0, tables, [n - 1], slot, store=False)]
             for _ in range(4):
                 self.step(rows)
-                if not ops.library_trials_pending():
+                if not products.trials_pending():
                     break
-            ops.settle_library_choices()
+            products.settle()
         if lengths:
             ops.prepare_library_adoption()
         torch.cuda.synchronize()

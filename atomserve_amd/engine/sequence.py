@@ -35,6 +35,18 @@ class SamplingParams:
     seed: Optional[int] = None
     ignore_eos: bool = False
 
+    def validated(self) -> "SamplingParams":
+        """Itself, or a ValueError that names the setting outside its range."""
+        if not self.temperature >= 0:
+            raise ValueError(f"temperature must be 0 (greedy) or positive, got {self.temperature}")
+        if self.top_k < 0:
+            raise ValueError(f"top_k must be 0 (all tokens) or positive, got {self.top_k}")
+        if not 0 < self.top_p <= 1:
+            raise ValueError(f"top_p must lie in (0, 1], got {self.top_p}")
+        if self.max_tokens < 1:
+            raise ValueError("max_tokens must be at least 1")
+        return self
+
 
 # The model card's settings for its two modes (reference atomserve/sequence.py:46-48).
 THINKING_PARAMS = SamplingParams(temperature=0.6, top_p=0.95, top_k=20)

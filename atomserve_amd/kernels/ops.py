@@ -47,32 +47,56 @@ def _ptr(t) -> int:
 
 # ---- weights in the order in which a wave reads them -------------------------------------------
 #
-# The few-rows products stream a weight matrix once per step.  `wave_order(w)` makes a second copy of
-# a bf16 matrix [R, K] (R % 16 == 0, K % 64 == 0) whose 16-byte pieces lie as a wave of those kernels
-# takes them, and hangs it on the tensor; the products that are handed `w` then read the copy (every
-# load instruction 1 KB in one piece, marked as not to be kept: 7 per cent less time for the 144
-# products of a decode step at Qwen3-8B sizes).  The library's products, the tile kernels and
-# everything else go on reading `w` itself.  Whoever changes `w` afterwards calls it again.
-WAVE_ORDER = "in_wave_order"
+# The few-rows and tile products stream a weight matrix once per step.  `Streamed(w)` holds a bf16
+# matrix [R, K] (R % 16 == 0, K % 64 == 0) a second time, its 16-byte pieces lying as a wave of those
+# kernels takes them; the products that are handed the `Streamed` read that copy (every load
+# instruction 1 KB in one piece, marked as not to be kept: 7 per cent less time for the 144 products of
+# a decode step at Qwen3-8B sizes), the library's products and everything else read the rows.  The
+# owner of the matrix (a part, the decoder for its head) owns the `Streamed` and with it the copy's
+# memory; whoever changes the rows in place afterwards calls `refresh()`.
 
 
-def wave_order(w):
-    """Attaches the copy in wave order to the bf16 matrix `w` on a GPU (and returns it); None, and
-    nothing attached, where the sizes or the dtype do not allow it."""
-    if w.dtype != BF16 or w.dim() != 2 or not w.is_cuda or not w.is_contiguous() or w.shape[0] % 16 or w.shape[1] % 64:
-        if hasattr(w, WAVE_ORDER):
-            delattr(w, WAVE_ORDER)
-        return None
-    copy = torch.empty_like(w)
-    call("as_wave_order", _ptr(w), _ptr(copy), w.shape[0], w.shape[1], _stream())
-    setattr(w, WAVE_ORDER, copy)
-    return copy
+class Streamed:
+    """A weight matrix as the products of this module read it: `rows`, the tensor [R, K] itself, and
+    `wave`, its copy in wave order, or None where the dtype or the sizes do not allow one or the owner
+    asked for none (`copy=False`: the copy's bytes are saved, decode steps stream the rows)."""
+
+    __slots__ = ("rows", "wave")
+
+    def __init__(self, rows, copy: bool = True):
+        self.rows, self.wave = rows, None
+        if copy:
+            self.refresh()
+
+    @staticmethod
+    def possible(w) -> bool:
+        return w.dtype == BF16 and w.dim() == 2 and w.is_cuda and w.is_contiguous() and w.shape[0] % 16 == 0 and w.shape[1] % 64 == 0
+
+    def refresh(self):
+        """Makes the copy (anew) from the rows as they are now; returns it, None where there can be none."""
+        if not self.possible(self.rows):
+            self.wave = None
+            return None
+        if self.wave is None:
+            self.wave = torch.empty_like(self.rows)
+        call("as_wave_order", _ptr(self.rows), _ptr(self.wave), self.rows.shape[0], self.rows.shape[1], _stream())
+        return self.wave
+
+    @property
+    def wave_bytes(self) -> int:
+        return 0 if self.wave is None else self.wave.numel() * self.wave.element_size()
+
+
+def _rows(w):
+    """The matrix itself of what a product was handed as its weights (a tensor, or a `Streamed`)."""
+    return w.rows if isinstance(w, Streamed) else w
 
 
 def _wave_ptr(w) -> int:
-    """The address of the copy of `w` in wave order, 0 if it has none."""
-    copy = getattr(w, WAVE_ORDER, None)
-    return 0 if copy is None else copy.data_ptr()
+    """The address of the copy in wave order of a product's weights, 0 if they have none."""
+    if isinstance(w, Streamed) and w.wave is not None:
+        return w.wave.data_ptr()
+    return 0
 
 
 def embed_gather(table, ids, out, scale: float = 1.0) -> None:
@@ -430,146 +454,73 @@ def _few_rows(rows: int, k: int, n: int, max_k=None, w=None) -> bool:
             and strips * rows * k * 2 <= SKINNY_TWO_MAX_ACT_BYTES)  # fmt: skip
 
 
-def gemm(a, w, out) -> None:
+def gemm(a, w, out, choices=None) -> None:
     """out[M, N] = a[M, K] @ w[N, K]^T.  fp32: own kernel (true fp32).  bf16: own kernel for few
-    rows, the library's matrix product otherwise; `out` may be bf16 or (few rows) fp32."""
+    rows, the library's matrix product otherwise; `out` may be bf16 or (few rows) fp32.
+    w: a tensor, or a `Streamed`.  choices: the `ProductChoices` that says which of the library's kernels
+    runs (a model's own; None: the one the process shares)."""
     _check(a, "a", (F32, BF16), (None, None))
     M, K = a.shape
-    _check(w, "w", a.dtype, (None, K))
-    N = w.shape[0]
+    rows = _rows(w)
+    _check(rows, "w", a.dtype, (None, K))
+    N = rows.shape[0]
     _check(out, "out", None, (M, N))
     if M == 0:
         return
     if a.dtype == F32:
         _check(out, "out", F32)
-        call("as_gemm_f32", _ptr(a), _ptr(w), _ptr(out), M, N, K, _stream())
+        call("as_gemm_f32", _ptr(a), _ptr(rows), _ptr(out), M, N, K, _stream())
         return
     if out.dtype not in (BF16, F32):
         raise KernelError(f"gemm: unsupported output dtype {out.dtype}")
     if _few_rows(M, K, N, w=w if out.dtype == BF16 else None):  # fp32 results (the head): no tile product to prefer
-        call("as_gemm_bf16_skinny", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), _DT[out.dtype], M, N, K, 0, _stream())
+        call("as_gemm_bf16_skinny", _ptr(a), _ptr(rows), _wave_ptr(w), _ptr(out), _DT[out.dtype], M, N, K, 0, _stream())
     else:
-        _library_gemm(a, w, out, M, N, K)
+        (choices or SHARED).gemm(a, w, out, M, N, K)
 
 
 # ---- the library's product, called directly -------------------------------------------------
 #
 # hipBLASLt through `csrc/blas.hip` instead of torch.mm: the same kernels for two thirds of the
-# time on the host.  For the row counts of LIBRARY_TUNED_ROWS (decode steps of 17 and more requests
-# are padded to a few row counts, which the capture of such a step adds here, and replayed thousands
-# of times) the library's first candidate is often not its fastest on this GPU, so the first calls
-# of such a shape try the candidates in turn, each on the weights of the layer that happens to call
-# (cold, as every decode step meets them), timed by events in place; when every candidate has run
-# LIBRARY_TRIALS_EACH times (the first run of a kernel is slow), or a capture begins, the fastest
-# stays.  The same is done for the row counts that `tune_library_rows` names (the token budget of a
-# step; lengths of prompts that a warm-up runs), and a product of any other row count above 64 takes
-# the kernel that the nearest tuned row count above it settled on: at 128 rows of Qwen3-8B sizes the
-# library's first candidates take 168 us a layer, the fastest of the first sixteen 132 us.
+# time on the host.  For the row counts that a `ProductChoices` is told to tune (decode steps of 17
+# and more requests are padded to a few row counts, which the capture of such a step names, and are
+# replayed thousands of times) the library's first candidate is often not its fastest on this GPU, so
+# the first calls of such a shape try the candidates in turn, each on the weights of the layer that
+# happens to call (cold, as every decode step meets them), timed by events in place; when every
+# candidate has run LIBRARY_TRIALS_EACH times (the first run of a kernel is slow), or a capture
+# begins, the fastest stays.  The same is done for the token budget of a step and for lengths of
+# prompts that a warm-up runs, and a product of any other row count above 64 takes the kernel that
+# the nearest tuned row count above it settled on: at 128 rows of Qwen3-8B sizes the library's first
+# candidates take 168 us a layer, the fastest of the first sixteen 132 us.
 LIBRARY_WORKSPACE_BYTES = 64 << 20
-LIBRARY_TUNED_ROWS = {32, 48, 64}
 LIBRARY_DECODE_ROWS = 64  # row counts up to here are decode steps' (padded to 32, 48 and 64)
 LIBRARY_TRIALS_EACH = 4
-_library = {"workspace": None, "choice": {}, "trials": {}, "fixed": False}
+_workspace = {}  # device index -> the library's scratch memory, one for the process (its calls follow one another)
 
-
-def fix_library_choices(fixed: bool = True) -> None:
-    """fixed: every shape not settled yet takes the library's first candidate (what torch.mm runs)
-    instead of timing the candidates, so that bfloat16 results are the same from process to process.
-    Choices already made stay (they were made under the setting of their time)."""
-    _library["fixed"] = bool(fixed)
-    if fixed:
-        _library["trials"].clear()
-
-
-def library_choices_fixed() -> bool:
-    return _library["fixed"]
-
-
-def library_choices() -> dict:
-    """(rows, columns, width, output dtype) -> the candidate that runs, for every shape settled so far
-    (-1: torch's own call; OWN_CANDIDATE + strips: this package's tile product); enough to reproduce a
-    run's products."""
-    return dict(_library["choice"])
-
-
-def _torch_gemm(a, w, out) -> None:
-    if out.dtype == BF16:
-        torch.mm(a, w.t(), out=out)
-    else:
-        out.copy_(torch.mm(a, w.t()))
-
-
-def _library_gemm(a, w, out, M, N, K) -> None:
-    state = _library
-    key = (M, N, K, out.dtype)
-    choice = state["choice"].get(key)
-    if choice is None:
-        capturing = torch.cuda.is_current_stream_capturing()
-        if state["workspace"] is None:
-            if capturing:  # nothing is allocated for good inside a capture: torch's own call this once
-                return _torch_gemm(a, w, out)
-            state["workspace"] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
-        trial = state["trials"].get(key)
-        if trial is None:
-            count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
-            if count == 0:
-                choice = state["choice"][key] = -1  # the library offers nothing for this shape through this door
-            elif state["fixed"] or (count == 1 and not _own_candidates(M, N, K, out.dtype, w)):
-                choice = state["choice"][key] = 0  # the library's first candidate, which is what torch.mm runs
-            elif M not in LIBRARY_TUNED_ROWS:
-                choice = _choice_of_tuned_rows(M, N, K, out.dtype)  # a prompt of any length: what its bucket settled on
-                if choice is None:
-                    choice = 0  # nothing settled yet: the first candidate for now, asked again at the next call
-                else:
-                    state["choice"][key] = choice
-            else:
-                ids = list(range(count)) + _own_candidates(M, N, K, out.dtype, w)
-                trial = state["trials"][key] = {"count": len(ids), "ids": ids, "runs": []}
-        if trial is not None:
-            if not capturing and not _tried_enough(trial):
-                trial["last"] = (a, w, out)
-                _trial_run(trial, a, w, out, M, N, K)
-                return
-            choice = state["choice"][key] = _fastest_of(state["trials"].pop(key))
-    if choice < 0:
-        return _torch_gemm(a, w, out)
-    if choice >= OWN_CANDIDATE and not _wave_ptr(w):
-        choice = 0  # chosen on weights that had a copy in wave order; these have none
-    _library_call(a, w, out, M, N, K, choice)
-
-
-def _choice_of_tuned_rows(M, N, K, dtype):
-    """For a product of a row count that is not tuned itself: the kernel that the nearest tuned row
-    count above it (of more than 64 rows: a prompt's, not a decode step's) settled on for the same
-    weights, as a candidate of this shape; None while that one has not settled, or there is none."""
-    above = [rows for rows in LIBRARY_TUNED_ROWS if rows >= M and rows > LIBRARY_DECODE_ROWS]
-    if not above:
-        return None
-    tuned = min(above)
-    settled = _library["choice"].get((tuned, N, K, dtype))
-    if settled is None:
-        return None
-    if settled < 0:
-        return 0
-    if settled >= OWN_CANDIDATE:  # this package's tile kernel: for this row count too if it takes it, else the library's first
-        return settled if settled in _own_candidates(M, N, K, dtype, None) else 0
-    index = entry("as_blas_candidate_index")(tuned, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, settled)
-    place = entry("as_blas_adopt")(M, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, index)
-    return place if place >= 0 else 0
-
-
-def prepare_library_adoption() -> bool:
-    """Pays the library's one-time cost of finding a kernel by its number (a third of a second) now, not
-    at the first prompt of a length that was not tuned.  False while no shape has been planned."""
-    return bool(entry("as_blas_prepare_adoption")())
-
-
-# Beside the library's candidates a trial may time this package's plain tile product (17 to 128 rows, K in
+# Beside the library's candidates a trial may time this package's plain tile product (9 to 128 rows, K in
 # chunks of 256, bf16 out, weights with a copy in wave order) with tiles of 2 and of 4 strips: for qkv
 # of Qwen3-8B sizes it takes 12.7 / 14.8 / 16.3 us at 32 / 48 / 64 rows against the library's best 14.7 /
 # 17.3 / 17.6; for the 4,096 columns of o the library wins at 32 to 64 rows.  Such a candidate's number
 # is OWN_CANDIDATE + its strips.
 OWN_CANDIDATE = 1000
+
+
+def _library_workspace(device):
+    """The library's scratch memory on `device`; None inside a capture that finds none yet (nothing is
+    allocated for good there)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    space = _workspace.get(index)
+    if space is None and not torch.cuda.is_current_stream_capturing():
+        space = _workspace[index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return space
+
+
+def _torch_gemm(a, w, out) -> None:
+    w = _rows(w)
+    if out.dtype == BF16:
+        torch.mm(a, w.t(), out=out)
+    else:
+        out.copy_(torch.mm(a, w.t()))
 
 
 def _own_candidates(M, N, K, dtype, w) -> list:
@@ -585,11 +536,125 @@ def _library_call(a, w, out, M, N, K, candidate) -> None:
     if candidate >= OWN_CANDIDATE:
         if not _wave_ptr(w) or out.dtype != BF16:
             raise KernelError("the tile product was chosen for weights with a copy in wave order and bf16 results")
-        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), 0, _DT[BF16], M, N, K, 0, 0,
+        call("as_gemm_bf16_tile", _ptr(a), _ptr(_rows(w)), _wave_ptr(w), _ptr(out), 0, _DT[BF16], M, N, K, 0, 0,
              candidate - OWN_CANDIDATE, _stream())  # fmt: skip
         return
-    call("as_blas_gemm", _ptr(a), _ptr(w), _ptr(out), _DT[out.dtype], M, N, K, candidate,
-         _ptr(_library["workspace"]), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip
+    call("as_blas_gemm", _ptr(a), _ptr(_rows(w)), _ptr(out), _DT[out.dtype], M, N, K, candidate,
+         _ptr(_library_workspace(a.device)), LIBRARY_WORKSPACE_BYTES, _stream())  # fmt: skip
+
+
+def prepare_library_adoption() -> bool:
+    """Pays the library's one-time cost of finding a kernel by its number (a third of a second) now, not
+    at the first prompt of a length that was not tuned.  False while no shape has been planned."""
+    return bool(entry("as_blas_prepare_adoption")())
+
+
+class ProductChoices:
+    """Which kernel runs for each shape of the matrix products that the few-rows kernels leave over: one
+    of the library's candidates or one of this package's tile products, settled by timed trials for the
+    row counts it is told to tune, or always the library's first (`fixed`).  A model owns one (its parts
+    hand it to `gemm`), so what is chosen on one model's weights, which row counts are tuned and whether
+    choices are fixed belong to that model's engine or tool and to no other in the process; calls that
+    name none share `SHARED`."""
+
+    def __init__(self, fixed: bool = False):
+        self.fixed = bool(fixed)
+        self.choice = {}  # (rows, columns, width, output dtype) -> candidate
+        self.trials = {}  # the same key -> a trial under way
+        self.tuned_rows = {32, 48, 64}
+
+    def fix(self, fixed: bool = True) -> None:
+        """fixed: every shape not settled yet takes the library's first candidate (what torch.mm runs)
+        instead of timing the candidates, so that bfloat16 results are the same from process to process.
+        Choices already made stay (they were made under the setting of their time)."""
+        self.fixed = bool(fixed)
+        if fixed:
+            self.trials.clear()
+
+    def chosen(self) -> dict:
+        """(rows, columns, width, output dtype) -> the candidate that runs, for every shape settled so far
+        (-1: torch's own call; OWN_CANDIDATE + strips: this package's tile product); enough to reproduce a
+        run's products."""
+        return dict(self.choice)
+
+    def tune_rows(self, rows: int) -> None:
+        """Also try the candidates for products of this many rows: a row count that comes again and
+        again, like the token budget of the steps that carry a portion of a prompt."""
+        self.tuned_rows.add(int(rows))
+
+    def trials_pending(self) -> bool:
+        """Whether some shape is still trying candidates (a warm-up may then run once more)."""
+        return bool(self.trials)
+
+    def gemm(self, a, w, out, M, N, K) -> None:
+        key = (M, N, K, out.dtype)
+        choice = self.choice.get(key)
+        if choice is None:
+            capturing = torch.cuda.is_current_stream_capturing()
+            if _library_workspace(a.device) is None:
+                return _torch_gemm(a, w, out)  # inside a capture, before any call outside one: torch's own call this once
+            trial = self.trials.get(key)
+            if trial is None:
+                count = entry("as_blas_plan")(M, N, K, _DT[out.dtype], LIBRARY_WORKSPACE_BYTES)
+                if count == 0:
+                    choice = self.choice[key] = -1  # the library offers nothing for this shape through this door
+                elif self.fixed or (count == 1 and not _own_candidates(M, N, K, out.dtype, w)):
+                    choice = self.choice[key] = 0  # the library's first candidate, which is what torch.mm runs
+                elif M not in self.tuned_rows:
+                    choice = self._choice_of_tuned_rows(M, N, K, out.dtype)  # a prompt of any length: what its bucket settled on
+                    if choice is None:
+                        choice = 0  # nothing settled yet: the first candidate for now, asked again at the next call
+                    else:
+                        self.choice[key] = choice
+                else:
+                    ids = list(range(count)) + _own_candidates(M, N, K, out.dtype, w)
+                    trial = self.trials[key] = {"count": len(ids), "ids": ids, "runs": []}
+            if trial is not None:
+                if not capturing and not _tried_enough(trial):
+                    trial["last"] = (a, w, out)
+                    _trial_run(trial, a, w, out, M, N, K)
+                    return
+                choice = self.choice[key] = _fastest_of(self.trials.pop(key))
+        if choice < 0:
+            return _torch_gemm(a, w, out)
+        if choice >= OWN_CANDIDATE and not _wave_ptr(w):
+            choice = 0  # chosen on weights that had a copy in wave order; these have none
+        _library_call(a, w, out, M, N, K, choice)
+
+    def _choice_of_tuned_rows(self, M, N, K, dtype):
+        """For a product of a row count that is not tuned itself: the kernel that the nearest tuned row
+        count above it (of more than 64 rows: a prompt's, not a decode step's) settled on for the same
+        weights, as a candidate of this shape; None while that one has not settled, or there is none."""
+        above = [rows for rows in self.tuned_rows if rows >= M and rows > LIBRARY_DECODE_ROWS]
+        if not above:
+            return None
+        tuned = min(above)
+        settled = self.choice.get((tuned, N, K, dtype))
+        if settled is None:
+            return None
+        if settled < 0:
+            return 0
+        if settled >= OWN_CANDIDATE:  # this package's tile kernel: for this row count too if it takes it, else the library's first
+            return settled if settled in _own_candidates(M, N, K, dtype, None) else 0
+        index = entry("as_blas_candidate_index")(tuned, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, settled)
+        place = entry("as_blas_adopt")(M, N, K, _DT[dtype], LIBRARY_WORKSPACE_BYTES, index)
+        return place if place >= 0 else 0
+
+    def settle(self) -> None:
+        """Ends every trial that is under way.  Called before a capture begins, so that the captured
+        launches are the ones later replays should make.  A shape that a pass meets once (the head)
+        has not come round often enough by then: the rest of its runs are made here, on the operands
+        of its last call."""
+        for key in list(self.trials):
+            trial = self.trials.pop(key)
+            a, w, out = trial["last"]
+            while not _tried_enough(trial):
+                _trial_run(trial, a, w, out, *key[:3])
+            torch.cuda.current_stream().synchronize()
+            self.choice[key] = _fastest_of(trial)
+
+
+SHARED = ProductChoices()  # for products whose caller names no choices of its own (tools, tests, toy parts)
 
 
 def _tried_enough(trial) -> bool:
@@ -609,32 +674,6 @@ def _trial_run(trial, a, w, out, M, N, K) -> None:
         return
     end.record()
     trial["runs"].append((candidate, start, end))
-
-
-def tune_library_rows(rows: int) -> None:
-    """Also try the candidates for products of this many rows: a row count that comes again and
-    again, like the token budget of the steps that carry a portion of a prompt."""
-    LIBRARY_TUNED_ROWS.add(int(rows))
-
-
-def library_trials_pending() -> bool:
-    """Whether some shape is still trying candidates (a warm-up may then run once more)."""
-    return bool(_library["trials"])
-
-
-def settle_library_choices() -> None:
-    """Ends every trial that is under way.  Called before a capture begins, so that the captured
-    launches are the ones later replays should make.  A shape that a pass meets once (the head)
-    has not come round often enough by then: the rest of its runs are made here, on the operands
-    of its last call."""
-    state = _library
-    for key in list(state["trials"]):
-        trial = state["trials"].pop(key)
-        a, w, out = trial["last"]
-        while not _tried_enough(trial):
-            _trial_run(trial, a, w, out, *key[:3])
-        torch.cuda.current_stream().synchronize()
-        state["choice"][key] = _fastest_of(trial)
 
 
 def _fastest_of(trial) -> int:
@@ -713,14 +752,15 @@ def gemm_split(a, w, plan=None):
     whoever takes them adds them up (`rmsnorm(..., split_sums=)`).  bf16, 17 to 128 rows."""
     _check(a, "a", BF16, (None, None))
     M, K = a.shape
-    _check(w, "w", BF16, (None, K))
-    N = w.shape[0]
+    rows = _rows(w)
+    _check(rows, "w", BF16, (None, K))
+    N = rows.shape[0]
     plan = plan or gemm_split_plan(M, N, K, a.dtype)
     if plan is None:
         raise KernelError(f"gemm_split: {M} rows, {K} -> {N} have no kernel")
     strips, splits = plan
     sums = torch.empty((splits, M, N), dtype=F32, device=a.device)
-    call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _wave_ptr(w), 0, _ptr(sums), _DT[F32], M, N, K, 0, splits, strips, _stream())
+    call("as_gemm_bf16_tile", _ptr(a), _ptr(rows), _wave_ptr(w), 0, _ptr(sums), _DT[F32], M, N, K, 0, splits, strips, _stream())
     return sums
 
 
@@ -736,7 +776,7 @@ def _gated_two_tiles(rows: int, k: int, w) -> bool:
         and k <= SKINNY_TWO_MAX_K and k % 8 == 0  # fmt: skip
 
 
-def gemm_silu_mul(a, w, out) -> None:
+def gemm_silu_mul(a, w, out, choices=None) -> None:
     """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for w[2 I, K]: the gate and up products and
     the activation.  bf16 with few rows: one kernel, the products rounded to bf16 before the
     activation exactly as the two-kernel path does; otherwise the product, then the activation."""
@@ -744,18 +784,19 @@ def gemm_silu_mul(a, w, out) -> None:
     M, K = a.shape
     _check(out, "out", a.dtype, (M, None))
     inter = out.shape[1]
-    _check(w, "w", a.dtype, (2 * inter, K))
+    rows = _rows(w)
+    _check(rows, "w", a.dtype, (2 * inter, K))
     if M == 0:
         return
     if a.dtype == BF16 and (_few_rows(M, K, inter, GATED_MAX_K, w=w) or _gated_two_tiles(M, K, w)):
-        call("as_gemm_bf16_gated", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), M, inter, K, _stream())
+        call("as_gemm_bf16_gated", _ptr(a), _ptr(rows), _wave_ptr(w), _ptr(out), M, inter, K, _stream())
         return
     if _tile_rows(M, K, a.dtype):
-        call("as_gemm_bf16_tile", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0,
+        call("as_gemm_bf16_tile", _ptr(a), _ptr(rows), _wave_ptr(w), _ptr(out), 0, _DT[BF16], M, inter, K, 1, 0,
              _gated_tile_strips(M, inter), _stream())  # fmt: skip
         return
     gate_up = torch.empty((M, 2 * inter), dtype=a.dtype, device=a.device)
-    gemm(a, w, gate_up)
+    gemm(a, w, gate_up, choices)
     silu_mul(gate_up, out)
 
 
@@ -784,15 +825,16 @@ def gemm_link(a, w, x, gain, scaled, ssq) -> None:
     a, w bf16; gain fp32 [N]."""
     _check(a, "a", BF16, (None, None))
     M, K = a.shape
-    _check(w, "w", BF16, (None, K))
-    N = w.shape[0]
+    rows = _rows(w)
+    _check(rows, "w", BF16, (None, K))
+    N = rows.shape[0]
     if not gemm_link_supported(M, N, K, a.dtype):
         raise KernelError(f"gemm_link: {M} rows, {K} -> {N} have no fused kernel")
     _check(x, "x", F32, (M, N))
     _check(gain, "gain", F32, (N,))
     _check(scaled, "scaled", BF16, (M, N))
     _check(ssq, "ssq", F32, (M, -(-N // 16)))
-    call("as_gemm_bf16_link", _ptr(a), _ptr(w), _wave_ptr(w), _ptr(x), _ptr(gain), _ptr(scaled), _ptr(ssq), M, N, K,
+    call("as_gemm_bf16_link", _ptr(a), _ptr(rows), _wave_ptr(w), _ptr(x), _ptr(gain), _ptr(scaled), _ptr(ssq), M, N, K,
          _stream())  # fmt: skip
 
 
@@ -805,10 +847,11 @@ def gemm_scaled(scaled, ssq, eps, w, out, gated=False) -> None:
     _check(ssq, "ssq", F32, (M, -(-K // 16)))
     _check(out, "out", BF16, (M, None))
     N = out.shape[1]
-    _check(w, "w", BF16, (2 * N if gated else N, K))
+    rows = _rows(w)
+    _check(rows, "w", BF16, (2 * N if gated else N, K))
     if not gemm_link_supported(M, K, 8, BF16):
         raise KernelError(f"gemm_scaled: {M} rows of width {K} have no fused kernel")
-    call("as_gemm_bf16_scaled", _ptr(scaled), _ptr(ssq), ssq.shape[1], float(eps), _ptr(w), _wave_ptr(w), _ptr(out), M, N, K,
+    call("as_gemm_bf16_scaled", _ptr(scaled), _ptr(ssq), ssq.shape[1], float(eps), _ptr(rows), _wave_ptr(w), _ptr(out), M, N, K,
          int(bool(gated)), _stream())  # fmt: skip
 
 

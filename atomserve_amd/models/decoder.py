@@ -11,11 +11,14 @@ from atomserve_amd.parts.plan import ModelPlan
 
 
 class DecoderModel:
-    def __init__(self, plan: ModelPlan, dtype: torch.dtype, device):
+    def __init__(self, plan: ModelPlan, dtype: torch.dtype, device, stream_copies: bool = True):
+        """stream_copies: keep the matrices that decode steps stream a second time, in the order their
+        kernels read them (`ops.Streamed`): faster decode steps for the weights' bytes again."""
         if dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"compute dtype must be float32 or bfloat16, got {dtype}")
         self.plan = plan
-        self.env = BuildEnv(dtype=dtype, device=torch.device(device))
+        self.env = BuildEnv(dtype=dtype, device=torch.device(device), stream_copies=bool(stream_copies),
+                            products=ops.ProductChoices())  # fmt: skip
         self.blocks = [build("arrangement", spec, self.env) for spec in plan.layers]
         self.final_norm = build("norm", plan.final_norm, self.env)
         for r in plan.run:
@@ -47,7 +50,7 @@ class DecoderModel:
         """Hand every part its tensors, by the names of `weight_decls`."""
         self.embed_weight = tensors["embed.weight"]
         self.head_weight = self.embed_weight if self.plan.tied_head else tensors["head.weight"]
-        ops.wave_order(self.head_weight)  # the head's product streams it at every decode step
+        self.head = ops.Streamed(self.head_weight, self.env.stream_copies)  # the head's product streams it at every decode step
         for i, block in enumerate(self.blocks):
             for part_name, part in block.parts().items():
                 prefix = f"layers.{i}.{part_name}."
@@ -60,6 +63,12 @@ class DecoderModel:
         """Bytes of all distinct tensors (a tied head counts once)."""
         seen = {t.data_ptr(): t.numel() * t.element_size() for t in self._tensors.values()}
         return sum(seen.values())
+
+    @property
+    def num_stream_copy_bytes(self) -> int:
+        """Bytes of the copies in wave order that the parts and the head keep beside the tensors."""
+        owned = [self.head] + [w for block in self.blocks for part in block.parts().values() for w in part.streamed()]
+        return sum(w.wave_bytes for w in owned)
 
     # ---- caches ---------------------------------------------------------------------
     def cache_requests(self) -> dict:
@@ -107,7 +116,7 @@ class DecoderModel:
             raise ValueError(f"the logits of this step are float32 {(n, p.vocab_size)}, the buffer is {tuple(logits.shape)}")
         if n:
             hf = self.final_norm.forward(x, delta, rows=step.logits_rows, update_residual=False)
-            ops.gemm(hf, self.head_weight, logits)
+            ops.gemm(hf, self.head, logits, self.env.products)
             if p.logit_scale != 1.0 or p.logit_softcap > 0.0:
                 ops.logits_finish(logits, p.logit_scale, p.logit_softcap)
         return logits

@@ -68,8 +68,12 @@ class Attention(Mixer):
 
     def bind(self, tensors: dict) -> None:
         super().bind(tensors)
-        for w in (self.qkv_weight, self.o_weight):
-            ops.wave_order(w)  # what the few-rows products of a decode step stream, where the sizes allow
+        # what the products of a decode step stream: the matrices with their copies in wave order
+        self.qkv = ops.Streamed(self.qkv_weight, self.env.stream_copies)
+        self.o = ops.Streamed(self.o_weight, self.env.stream_copies)
+
+    def streamed(self) -> list:
+        return [self.qkv, self.o]
 
     def cache_request(self):
         s = self.spec
@@ -88,9 +92,9 @@ class Attention(Mixer):
         H, KV, D = s.num_heads, s.num_kv_heads, s.head_dim
         qkv = torch.empty((T, (H + 2 * KV) * D), dtype=env.dtype, device=device)
         if pending:
-            h.gemm(self.qkv_weight, qkv)
+            h.gemm(self.qkv, qkv)
         else:
-            ops.gemm(h, self.qkv_weight, qkv)
+            ops.gemm(h, self.qkv, qkv, env.products)
         cos_sin = self.position.prepare(step) if self.position is not None else None
         eps = s.qk_norm.eps if s.qk_norm is not None else 0.0
         rotary = 2 * cos_sin.shape[1] if cos_sin is not None else 0
@@ -112,15 +116,15 @@ class Attention(Mixer):
             out = torch.empty((T, H, D), dtype=env.dtype, device=device)
             self.attend(q, out, step, cache)
         if residual is not None and next_norm is not None:
-            link = next_norm.absorb(out.view(T, H * D), self.o_weight, residual)
+            link = next_norm.absorb(out.view(T, H * D), self.o, residual)
             if link is not None:
                 return link
             if next_norm.takes_split_sums:
                 plan = ops.gemm_split_plan(T, s.hidden_size, out.view(T, H * D).shape[1], env.dtype)
                 if plan is not None:
-                    return SplitSums(ops.gemm_split(out.view(T, H * D), self.o_weight, plan))
+                    return SplitSums(ops.gemm_split(out.view(T, H * D), self.o, plan))
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=device)
-        ops.gemm(out.view(T, H * D), self.o_weight, y)
+        ops.gemm(out.view(T, H * D), self.o, y, env.products)
         return y
 
     def attend(self, q, out, step, cache) -> None:

@@ -77,6 +77,11 @@ class Part:
         for name, t in tensors.items():
             setattr(self, name.replace(".", "_"), t)
 
+    def streamed(self) -> list:
+        """The `ops.Streamed` matrices this part owns (their copies in wave order are memory beside the
+        checkpoint's tensors, which the model reports); none for most parts."""
+        return []
+
 
 @dataclass
 class BuildEnv:
@@ -84,6 +89,12 @@ class BuildEnv:
 
     dtype: torch.dtype  # compute dtype: torch.bfloat16 or torch.float32
     device: torch.device
+    # whether matrices that decode steps stream are kept a second time in the order their kernels read
+    # them (faster steps for the weights' bytes again); a part asks `ops.Streamed(w, env.stream_copies)`
+    stream_copies: bool = True
+    # which of the library's kernels the model's matrix products run (`ops.ProductChoices`): the model's own
+    # object, which its parts hand to `ops.gemm`; None: the one the process shares
+    products: Any = None
 
 
 class PendingNorm:

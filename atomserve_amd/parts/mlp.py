@@ -26,26 +26,30 @@ class GatedMLP(FeedForward):
 
     def bind(self, tensors: dict) -> None:
         super().bind(tensors)
-        for w in (self.gate_up_weight, self.down_weight):
-            ops.wave_order(w)  # what the few-rows products of a decode step stream, where the sizes allow
+        # what the products of a decode step stream: the matrices with their copies in wave order
+        self.gate_up = ops.Streamed(self.gate_up_weight, self.env.stream_copies)
+        self.down = ops.Streamed(self.down_weight, self.env.stream_copies)
+
+    def streamed(self) -> list:
+        return [self.gate_up, self.down]
 
     def forward(self, h, step, residual=None, next_norm=None):
         s, env = self.spec, self.env
         pending = isinstance(h, PendingNorm)
         T, device = (h.x.shape[0], h.x.device) if pending else (h.shape[0], h.device)
         act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=device)
-        if not (pending and h.gemm_gated(self.gate_up_weight, act, s.activation)):
-            ops.gemm_silu_mul(h.rows() if pending else h, self.gate_up_weight, act)
+        if not (pending and h.gemm_gated(self.gate_up, act, s.activation)):
+            ops.gemm_silu_mul(h.rows() if pending else h, self.gate_up, act, env.products)
         if residual is not None and next_norm is not None:
-            link = next_norm.absorb(act, self.down_weight, residual)
+            link = next_norm.absorb(act, self.down, residual)
             if link is not None:
                 return link
             if next_norm.takes_split_sums:
                 plan = ops.gemm_split_plan(T, s.hidden_size, act.shape[1], env.dtype)
                 if plan is not None:
-                    return SplitSums(ops.gemm_split(act, self.down_weight, plan))
+                    return SplitSums(ops.gemm_split(act, self.down, plan))
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=device)
-        ops.gemm(act, self.down_weight, y)
+        ops.gemm(act, self.down, y, env.products)
         return y
 
 

@@ -210,12 +210,12 @@ def load_weights(model_dir: str, model, arch, config) -> dict:
         return bind_checkpoint(model, arch, config, SafetensorsSource(model_dir, stack), where=f"in {model_dir}")
 
 
-def load_model(model_dir: str, dtype: torch.dtype, device):
+def load_model(model_dir: str, dtype: torch.dtype, device, stream_copies: bool = True):
     """config.json -> architecture -> plan -> model with its weights: (model, arch, config)."""
     from atomserve_amd.config.registry import load_model_config
     from atomserve_amd.models.decoder import DecoderModel
 
     arch, config = load_model_config(model_dir)
-    model = DecoderModel(arch.build_plan(config), dtype, device)
+    model = DecoderModel(arch.build_plan(config), dtype, device, stream_copies=stream_copies)
     load_weights(model_dir, model, arch, config)
     return model, arch, config

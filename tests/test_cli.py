@@ -80,3 +80,19 @@ def test_the_reserve_of_a_step_grows_with_its_budget_and_the_vocabulary():
     small, large = step_reserve_bytes(plan, 512, 32), step_reserve_bytes(plan, 8192, 32)
     assert 2**30 < small < large < 8 * 2**30
     assert step_reserve_bytes(build_plan(Qwen3Config(**{**cfg, "vocab_size": 1000})), 512, 32) < small
+
+
+def test_limits_that_contradict_each_other_are_a_message():
+    """A token budget smaller than the number of running requests (one decoded token each) or a pool of no
+    pages ends with a message that names it, as an exit of the program, not as a traceback."""
+    block_bytes = 28 * 2 * 8 * 128 * 2 * 16
+    with pytest.raises(SystemExit, match="max_num_batched_tokens"):
+        engine_config_for(build_parser().parse_args(["m", "--max-batched-tokens", "8", "--max-num-seqs", "16"]), block_bytes, 40960)
+    with pytest.raises(SystemExit, match="positive"):
+        engine_config_for(build_parser().parse_args(["m", "--block-size", "0"]), block_bytes, 40960)
+    with pytest.raises(SystemExit, match="no room for a single KV block"):
+        engine_config_for(build_parser().parse_args(["m", "--kv-mem-gb", "0.000001"]), block_bytes, 40960)
+    # a --max-model-len above what pool and model allow is cut down to it, not an error
+    cut = engine_config_for(build_parser().parse_args(["m", "--kv-mem-gb", "1", "--max-model-len", "1000000"]), block_bytes, 40960)
+    assert cut.max_model_len == cut.num_blocks * 16
+    assert build_parser().parse_args(["m", "--no-stream-copies"]).no_stream_copies is True

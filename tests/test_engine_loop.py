@@ -99,6 +99,10 @@ def test_submit_validates():
         e.submit([1] * 64, GREEDY)
     with pytest.raises(ValueError, match="max_tokens"):
         e.submit([1], SamplingParams(max_tokens=0))
+    for bad, named in ((dict(temperature=-0.5), "temperature"), (dict(top_p=0.0), "top_p"), (dict(top_p=1.5), "top_p"),
+                       (dict(top_k=-1), "top_k"), (dict(temperature=float("nan")), "temperature")):  # fmt: skip
+        with pytest.raises(ValueError, match=named):
+            e.submit([1], SamplingParams(**bad))
     with pytest.raises(ValueError, match="vocabulary"):
         e.submit([1, 1000], GREEDY)
 

@@ -367,9 +367,14 @@ def test_every_candidate_of_the_library_gives_the_product(ops):
         out.zero_()
         ops.gemm(a, w, out)
         assert close_bf16(out, ref, scale=math.sqrt(K))
-    assert (M, N, K, BF16) in ops._library["choice"]
-    ops.settle_library_choices()  # and whatever other tests left half tried
-    assert not ops.library_trials_pending()
+    assert (M, N, K, BF16) in ops.SHARED.chosen()
+    ops.SHARED.settle()  # and whatever other tests left half tried
+    assert not ops.SHARED.trials_pending()
+    # choices are a model's own: another object starts with none, and fixed takes the first candidate
+    mine = ops.ProductChoices(fixed=True)
+    out.zero_()
+    ops.gemm(a, w, out, mine)
+    assert close_bf16(out, ref, scale=math.sqrt(K)) and mine.chosen() == {(M, N, K, BF16): 0}
 
 
 def test_a_product_of_any_row_count_takes_what_the_tuned_count_above_it_chose(ops):
@@ -384,40 +389,36 @@ def test_a_product_of_any_row_count_takes_what_the_tuned_count_above_it_chose(op
     a = torch.randn(M, K, device=DEV).to(BF16)
     out = torch.empty(M, N, dtype=BF16, device=DEV)
     number = lambda rows, place: entry("as_blas_candidate_index")(rows, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, place)
-    was_fixed = ops.library_choices_fixed()
-    ops.fix_library_choices(False)
-    ops.tune_library_rows(tuned)
-    try:
-        ops.gemm(a, w, out)  # nothing settled above 100 rows: the first candidate, and no decision
-        assert close_bf16(out, pk.gemm(a, w), scale=math.sqrt(K)) and (M, N, K, BF16) not in ops.library_choices()
-        big = torch.randn(tuned, K, device=DEV).to(BF16)
-        big_out = torch.empty(tuned, N, dtype=BF16, device=DEV)
-        while (tuned, N, K, BF16) not in ops.library_choices():
-            ops.gemm(big, w, big_out)
-        chosen = ops.library_choices()[(tuned, N, K, BF16)]
-        out.fill_(float("nan"))
-        ops.gemm(a, w, out)
-        assert close_bf16(out, pk.gemm(a, w), scale=math.sqrt(K))
-        mine = ops.library_choices()[(M, N, K, BF16)]
-        assert number(M, mine) == number(tuned, chosen) or (mine == 0 and entry("as_blas_adopt")(M, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, chosen)) < 0)
-        # a kernel that this shape's own list does not hold is added to it, once
-        count = entry("as_blas_plan")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)
-        for place in range(entry("as_blas_plan")(tuned, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)):
-            at = entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, place))
-            assert at < 0 or number(M + 1, at) == number(tuned, place)
-            assert at == entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, place))
-        grown = entry("as_blas_plan")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)
-        assert grown >= count
-        a1 = torch.randn(M + 1, K, device=DEV).to(BF16)
-        for place in range(count, grown):  # the adopted ones give the product too
-            o1 = torch.zeros(M + 1, N, dtype=BF16, device=DEV)
-            ops._library_call(a1, w, o1, M + 1, N, K, place)
-            assert close_bf16(o1, pk.gemm(a1, w), scale=math.sqrt(K)), place
-        assert entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, -1) < 0
-        assert ops.prepare_library_adoption()  # the look-up by number that a warm-up makes ahead of serving
-    finally:
-        ops.LIBRARY_TUNED_ROWS.discard(tuned)
-        ops.fix_library_choices(was_fixed)
+    choices = ops.ProductChoices()
+    choices.tune_rows(tuned)
+    ops.gemm(a, w, out, choices)  # nothing settled above 100 rows: the first candidate, and no decision
+    assert close_bf16(out, pk.gemm(a, w), scale=math.sqrt(K)) and (M, N, K, BF16) not in choices.chosen()
+    big = torch.randn(tuned, K, device=DEV).to(BF16)
+    big_out = torch.empty(tuned, N, dtype=BF16, device=DEV)
+    while (tuned, N, K, BF16) not in choices.chosen():
+        ops.gemm(big, w, big_out, choices)
+    chosen = choices.chosen()[(tuned, N, K, BF16)]
+    out.fill_(float("nan"))
+    ops.gemm(a, w, out, choices)
+    assert close_bf16(out, pk.gemm(a, w), scale=math.sqrt(K))
+    mine = choices.chosen()[(M, N, K, BF16)]
+    assert number(M, mine) == number(tuned, chosen) or (mine == 0 and entry("as_blas_adopt")(M, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, chosen)) < 0)
+    # a kernel that this shape's own list does not hold is added to it, once
+    count = entry("as_blas_plan")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)
+    for place in range(entry("as_blas_plan")(tuned, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)):
+        at = entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, place))
+        assert at < 0 or number(M + 1, at) == number(tuned, place)
+        assert at == entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, number(tuned, place))
+    grown = entry("as_blas_plan")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES)
+    assert grown >= count
+    a1 = torch.randn(M + 1, K, device=DEV).to(BF16)
+    for place in range(count, grown):  # the adopted ones give the product too
+        o1 = torch.zeros(M + 1, N, dtype=BF16, device=DEV)
+        ops._library_call(a1, w, o1, M + 1, N, K, place)
+        assert close_bf16(o1, pk.gemm(a1, w), scale=math.sqrt(K)), place
+    assert entry("as_blas_adopt")(M + 1, N, K, 1, ops.LIBRARY_WORKSPACE_BYTES, -1) < 0
+    assert ops.prepare_library_adoption()  # the look-up by number that a warm-up makes ahead of serving
+    assert (tuned, N, K, BF16) not in ops.SHARED.chosen() and tuned not in ops.SHARED.tuned_rows  # nobody else's business
 
 
 @pytest.mark.parametrize("M,N,K", [(48, 544, 1024), (9, 544, 1024), (12, 6144, 4096), (16, 1024, 2560), (128, 48, 256)])
@@ -429,32 +430,28 @@ def test_the_tile_product_is_a_candidate_beside_the_librarys(ops, M, N, K):
     a = torch.randn(M, K, device=DEV).to(BF16)
     w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(BF16)
     bare = w.clone()
-    assert ops._own_candidates(M, N, K, BF16, w) == []  # no copy yet
-    ops.wave_order(w)
+    assert ops._own_candidates(M, N, K, BF16, w) == [] and ops._own_candidates(M, N, K, BF16, ops.Streamed(w, copy=False)) == []
+    w = ops.Streamed(w)  # with its copy in wave order
     own = ops._own_candidates(M, N, K, BF16, w)
     assert own == [ops.OWN_CANDIDATE + 2, ops.OWN_CANDIDATE + 4]
     assert ops._own_candidates(M, N + 8, K, BF16, None) == [] and ops._own_candidates(8, N, K, BF16, None) == []
     assert ops._own_candidates(M, N, K + 64, BF16, None) == [] and ops._own_candidates(129, N, K, BF16, None) == []
-    ref = pk.gemm(a, w)
+    ref = pk.gemm(a, bare)
     key = (M, N, K, BF16)
-    kept = ops._library["choice"].get(key)
-    try:
-        for candidate in own:
-            out = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
-            ops._library_call(a, w, out, M, N, K, candidate)
+    for candidate in own:
+        choices = ops.ProductChoices()
+        choices.tune_rows(M)
+        out = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
+        ops._library_call(a, w, out, M, N, K, candidate)
+        assert close_bf16(out, ref, scale=1.0)
+        choices.gemm(a, w, out, M, N, K)  # makes the library's plan and workspace for this shape, and starts a trial
+        assert choices.trials[key]["ids"][-2:] == own  # this package's products are tried beside the library's
+        choices.trials.clear()
+        choices.choice[key] = candidate
+        for weights in (w, bare):
+            out.fill_(float("nan"))
+            choices.gemm(a, weights, out, M, N, K)
             assert close_bf16(out, ref, scale=1.0)
-            ops._library_gemm(a, w, out, M, N, K)  # makes the library's plan and workspace for this shape
-            ops._library["choice"][key] = candidate
-            for weights in (w, bare):
-                out.fill_(float("nan"))
-                ops._library_gemm(a, weights, out, M, N, K)
-                assert close_bf16(out, ref, scale=1.0)
-    finally:
-        ops._library["trials"].pop(key, None)
-        if kept is None:
-            ops._library["choice"].pop(key, None)
-        else:
-            ops._library["choice"][key] = kept
 
 
 def test_library_candidates_replay_from_a_graph(ops):
@@ -584,14 +581,16 @@ def test_weights_in_wave_order_give_the_same_products(ops, M, N, K):
     bit what it gives from rows (the same values reach the same lanes).  Sizes of both few-rows kernels,
     whole and partial workgroup rounds, one and two row tiles; sizes that take no copy go on as before."""
     torch.manual_seed(M * 7 + N)
-    w = (torch.randn(2 * N, K, device=DEV) / math.sqrt(K)).to(BF16)
-    copy = ops.wave_order(w)
+    values = (torch.randn(2 * N, K, device=DEV) / math.sqrt(K)).to(BF16)
+    w = ops.Streamed(values)
+    copy = w.wave
     if (2 * N) % 16 or K % 64:
-        assert copy is None and not hasattr(w, ops.WAVE_ORDER)
+        assert copy is None and w.wave_bytes == 0 and not ops.Streamed.possible(values)
         return
-    want = w.view(2 * N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous().view(2 * N, K)  # strip, step, half, lane / 16, lane % 16
-    assert torch.equal(copy, want) and getattr(w, ops.WAVE_ORDER) is copy
-    plain = w.clone()  # the same values without a copy
+    want = values.view(2 * N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous().view(2 * N, K)  # strip, step, half, lane / 16, lane % 16
+    assert torch.equal(copy, want) and w.rows is values and w.wave_bytes == values.numel() * 2
+    assert ops.Streamed(values, copy=False).wave is None  # the owner asked for none
+    plain = values.clone()  # the same values without a copy
     a = torch.randn(M, K, device=DEV).to(BF16)
 
     def both(run, *outs):
@@ -632,9 +631,15 @@ def test_weights_in_wave_order_give_the_same_products(ops, M, N, K):
         for gated in (False, True):
             both(lambda wt, out: ops.gemm_scaled(a, ssq, 1e-5, wt, out, gated=gated),
                  torch.empty(M, N if gated else 2 * N, dtype=BF16, device=DEV))
-    # a changed matrix takes a new copy; one that no longer qualifies loses it
-    w.mul_(2)
-    assert torch.equal(ops.wave_order(w), (want.float() * 2).to(BF16))
+    # a matrix changed in place takes its copy anew when its owner says so, and the products follow
+    values.mul_(2)
+    assert torch.equal(w.wave, want)  # stale until then
+    assert torch.equal(w.refresh(), (want.float() * 2).to(BF16)) and w.wave is copy
+    if ops._few_rows(M, K, 2 * N, w=w):
+        got, ref = torch.empty(M, 2 * N, dtype=BF16, device=DEV), torch.empty(M, 2 * N, dtype=BF16, device=DEV)
+        ops.gemm(a, w, got)
+        ops.gemm(a, values.clone(), ref)
+        assert torch.equal(got, ref)
 
 
 def test_gemm_link_refuses_what_it_cannot_do(ops):
@@ -1077,7 +1082,7 @@ def test_products_of_9_to_128_rows_in_tiles(ops, M, N, K):
     gated_ref = (lambda g: torch.nn.functional.silu(g[:, :N]) * g[:, N:])(ref.to(BF16).double())
     chunks = K // 256
     typical = float(ref.pow(2).mean().sqrt())
-    copy = ops.wave_order(w) if N % 16 == 0 else None  # the gated and the split variant also read weights in wave order
+    copy = ops.Streamed(w).wave if N % 16 == 0 else None  # the gated and the split variant also read weights in wave order
     for strips, wt in [(n, p) for n in (8, 6, 4, 2) for p in ([0] if copy is None else [0, copy.data_ptr()])]:
         out = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
         call("as_gemm_bf16_tile", a.data_ptr(), w.data_ptr(), wt, out.data_ptr(), 0, 1, M, N, K, 0, 0, strips, stream)
@@ -1104,11 +1109,13 @@ def test_products_of_9_to_128_rows_in_tiles(ops, M, N, K):
             run()  # ranges of equal length, or the last one shorter
             assert torch.allclose(sums.double().sum(0), ref[:, :N], atol=1e-3, rtol=1e-4), f"{splits} ranges, {strips} strips"
     # through the wrappers: the gated product, and split sums taken in by the norm
-    act = torch.empty(M, N, dtype=BF16, device=DEV)
-    ops.gemm_silu_mul(a, w, act)
-    assert torch.allclose(act.double(), gated_ref, atol=2e-2, rtol=2e-2)
+    for weights in (w, ops.Streamed(w)):  # from rows, and from the copy in wave order where the sizes allow one
+        act = torch.full((M, N), float("nan"), dtype=BF16, device=DEV)
+        ops.gemm_silu_mul(a, weights, act)
+        assert torch.allclose(act.double(), gated_ref, atol=2e-2, rtol=2e-2)
     if N % 4 == 0:
-        sums = ops.gemm_split(a, w[:N].contiguous())
+        sums = ops.gemm_split(a, ops.Streamed(w[:N].contiguous()))
+        assert torch.equal(sums, ops.gemm_split(a, w[:N].contiguous()))  # the same values reach the same lanes
         x = torch.randn(M, N, device=DEV)
         gain = (torch.randn(N, device=DEV) + 1).to(BF16)
         x1, x2 = x.clone(), x.clone()

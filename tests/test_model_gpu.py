@@ -711,3 +711,31 @@ def test_a_callers_own_graph_after_the_engines(setup):
     graph.replay()
     torch.cuda.synchronize()
     assert x.tolist() == [2.0] * 8
+
+
+def test_a_replay_step_that_cannot_run_changes_nothing(setup):
+    """A token outside the vocabulary, a wanted place outside its row, a request named twice, a step
+    without room: each raises before a page is taken, the requests that were alive keep what they held,
+    nobody new is alive, and the trace goes on to the plain model's logits."""
+    name, raw, weights, path, cache = setup
+    vocab = raw["vocab_size"]
+    ids = rc.random_ids(vocab, 40, seed=12)
+    replay = make_replay(path, "float32", 128, PAGE[name])
+    first = replay.step([{"id": "a", "tokens": ids[:20], "want": [19]}], [])
+    held = replay.manager.num_free
+    bad_steps = [
+        [{"id": "a", "tokens": ids[20:22], "want": [0]}, {"id": "b", "tokens": [1, vocab], "want": [1]}],
+        [{"id": "a", "tokens": ids[20:22], "want": [2]}],
+        [{"id": "b", "tokens": [1, 2], "want": [-1]}],
+        [{"id": "b", "tokens": [1], "want": []}, {"id": "b", "tokens": [2], "want": []}],
+        [{"id": "b", "tokens": [1] * 500, "want": []}],
+    ]
+    for entries in bad_steps:
+        with pytest.raises((ValueError, RuntimeError)):
+            replay.step(entries, [])
+        assert replay.manager.num_free == held and sorted(replay.live) == ["a"] and replay.live["a"][1] == 20
+    rest = replay.step([{"id": "a", "tokens": ids[20:], "want": [19]}], ["a"])
+    ref = rc.plain_rows(raw, weights, ids, {}, "a", False)
+    for got, place in ((first[0], 19), (rest[0], 39)):
+        assert float((got - ref[place]).abs().max()) <= rc.TOL_FLOAT32 * max(1.0, float(ref.abs().max()))
+    assert replay.manager.num_free == replay.manager.num_blocks and not replay.live

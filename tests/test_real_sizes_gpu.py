@@ -203,7 +203,6 @@ def test_layer_sizes_of_every_model_the_benchmark_names(size, dtype, products):
     picks, as serving does."""
     from atomserve_amd.config import Qwen3Config
     from atomserve_amd.engine.replay import Replay
-    from atomserve_amd.kernels import ops
 
     assert set(bench.SIZES) == {"0.6b", "1.7b", "4b", "8b", "14b", "32b"}  # a size added there is added here
     raw = Qwen3Config(**{**bench.SIZES[size], "num_layers": 2, "vocab_size": 5008}).to_dict()
@@ -211,14 +210,13 @@ def test_layer_sizes_of_every_model_the_benchmark_names(size, dtype, products):
     exact64 = {k: v.double() for k, v in exact.items()}
     requests, steps = trace_of_every_route(raw["vocab_size"])
     model = build(arch, config, exact if dtype == "float32" else stored, getattr(torch, dtype))
-    was_fixed = ops.library_choices_fixed()
-    try:
-        replay = Replay(None, dtype, rc.live_token_bound(steps), max_live=65, model=model, fixed_products=products == "first")
-        got = wanted_rows(replay, steps)
-        if products == "timed":  # the captured steps of 32 and 64 rows did settle on candidates of their own
-            assert {rows for rows, _, _, _ in ops.library_choices()} >= {32, 64} and not ops.library_trials_pending()
-    finally:
-        ops.fix_library_choices(was_fixed)
+    replay = Replay(None, dtype, rc.live_token_bound(steps), max_live=65, model=model, fixed_products=products == "first")
+    got = wanted_rows(replay, steps)
+    chosen = model.env.products.chosen()  # this model's own: no other engine of the process chose for it
+    if dtype == "bfloat16":
+        assert {rows for rows, _, _, _ in chosen} >= {32, 64} and not model.env.products.trials_pending()
+    if products == "first":
+        assert set(chosen.values()) <= {0, -1}
     assert replay.manager.num_free == replay.manager.num_blocks and len(got) == 65 + 66 + 3 + 2 * (64 + 32 + 16 + 12 + 8 + 3 + 1)
     assert sorted(n for n, _ in replay.runner.decode_graphs.graphs) == [1, 4, 8, 16, 32, 64]
     err, noise, scale = rc.Spread(), rc.Spread(), 0.0

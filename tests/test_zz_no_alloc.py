@@ -6,9 +6,12 @@ import ctypes
 import pytest
 import torch
 
+from tests import plain_kernels as pk
+
 pytestmark = pytest.mark.gpu
 
 P_, I_, F_ = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+TOL = {torch.float32: dict(atol=2e-5, rtol=1e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
 
 
 def static_entry():
@@ -60,6 +63,42 @@ def test_two_calls_in_a_row_match_the_entry_point_with_buffers(dtype):
                     D**-0.5, 0, part, P, stream)  # fmt: skip
         assert status == 0
         torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        # and both are the plain attention over the same pages (a fault the two entry points share would pass the line above)
+        plain = pk.paged_attention(q, k, v, torch.arange(n), positions, torch.arange(n), tables, D**-0.5)
+        assert torch.allclose(got.float(), plain, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_listed_tokens_of_rows_and_contexts_in_one_piece(dtype):
+    """The other ways to call it: some tokens of a step listed in an order of the caller's, each token
+    reading the block table of its row (portions of two requests), with the contexts cut into partitions
+    (the scratch array) and in one piece (no scratch at all); a window on top.  Against the plain
+    attention, and bit for bit against the entry point with buffers."""
+    from atomserve_amd.kernels import ops
+
+    fn = static_entry()
+    stream = torch.cuda.current_stream().cuda_stream
+    H, KV, D, bs = 6, 2, 32, 8
+    contexts = [330, 61]  # two requests; the step brings the last 5 tokens of the first and the last 3 of the second
+    q, k, v, tables, _ = case(dtype, 8, contexts, H, KV, D, bs, seed=9)
+    tables = tables[:2].contiguous()
+    positions = torch.tensor([325, 326, 327, 328, 329, 58, 59, 60], dtype=torch.int32, device="cuda")
+    tok_row = torch.tensor([0, 0, 0, 0, 0, 1, 1, 1], dtype=torch.int32, device="cuda")
+    items = torch.tensor([7, 2, 4, 5, 0], dtype=torch.int32, device="cuda")  # five of the eight, in no order
+    for window, part in ((0, 64), (0, 512), (40, 64)):
+        P = -(-max(contexts) // part)
+        got = torch.zeros_like(q)
+        status = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), 0 if dtype == torch.float32 else 1, items.data_ptr(), 5,
+                    positions.data_ptr(), tok_row.data_ptr(), tables.data_ptr(), tables.shape[1], got.data_ptr(), H, KV, D,
+                    bs, D**-0.5, window, part, P, stream)  # fmt: skip
+        assert status == 0 and (P == 1) == (part == 512)
+        torch.cuda.synchronize()
+        plain = pk.paged_attention(q, k, v, items, positions, tok_row, tables, D**-0.5, window)
+        assert torch.allclose(got.float(), plain, **TOL[dtype])  # the tokens not listed stay as they were: zero
+        want = torch.zeros_like(q)
+        ops.attn_single_query(q, k, v, items, positions, tok_row, tables, want, D**-0.5, window, max(contexts),
+                              part_size=part, force_generic=True)  # fmt: skip
         assert torch.equal(got, want)
 
 
