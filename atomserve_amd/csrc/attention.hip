@@ -674,11 +674,26 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 // s_waitcnt that only constrains the vector-memory counter (vmcnt: bits 3:0 and 15:14)
 #define PF_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
 
+// A step of few work items takes as long as its longest one (a portion of a prompt behind thousands of cached
+// tokens: a hundred workgroups of hundreds of rounds each, on a GPU with room for five hundred).  With `pieces` > 1
+// every work item comes as that many workgroups: an item of more than `piece_rounds` rounds of 64 keys is cut
+// along its keys into pieces of that many rounds (the last one, with the causal diagonal, may be shorter), each
+// piece leaves the maxima, sums and unnormalised outputs of its queries, and `attn_prefill_merge_kernel` puts them
+// together; a shorter item is its first workgroup's alone, as without the cut, and the others leave at once.
+struct PrefillSplit {
+  int pieces;        // workgroups per item; 1: no item is cut
+  int piece_rounds;  // rounds of a piece
+  int* cut;          // [items]: the pieces the item was cut into (1: not cut), for the merge
+  float* ml;         // [T, H, pieces, 2]: maximum (base 2, scaled) and sum
+  float* acc;        // [T, H, pieces, D]: unnormalised output
+};
+constexpr int PREFILL_MIN_PIECE_ROUNDS = 2;  // an item's last two rounds hold its own tokens: one piece
+
 template <int DC, int QT>  // D / 32; column tiles of 16 queries that a wave owns: 2, or 1 (see the launcher)
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ tiles, const int* __restrict__ block_tables, int table_width,
-    bf16* __restrict__ out, int H, int KV, int bs, float scale, int window, int units_z, int pass) {
+    bf16* __restrict__ out, int H, int KV, int bs, float scale, int window, int units_z, int pass, PrefillSplit split) {
   constexpr int D = DC * 32, DT = DC * 2;
   constexpr int PIECE = 64 * DC;  // 16-byte slots of a 16-key piece: 16 * D / 8
   typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
@@ -700,6 +715,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const int size = min(pass, (int)gridDim.x - first);
     if (block & 1) item = first + size - 1 - (item - first);
   }
+  int piece = 0;  // which of an item's workgroups this is
+  if (split.pieces > 1) {
+    piece = item % split.pieces;
+    item /= split.pieces;
+  }
   const int tile = item / per_tile, kvh = (item % per_tile) / units_z, bz = item % units_z;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -717,7 +737,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     wg_last = max(wg_last, pos0 + min(count, uq0 + WQ) - 1);
     wg_lo = min(wg_lo, window > 0 ? max(0, pos0 + uq0 - window + 1) : 0);
   }
-  if (wg_last < 0) return;  // uniform over the workgroup
+  if (wg_last < 0) {  // uniform over the workgroup
+    if (split.pieces > 1 && piece == 0 && threadIdx.x == 0) split.cut[item] = 1;
+    return;
+  }
+  bool partial = false;  // this workgroup leaves its share of a cut item for the merge
+  if (split.pieces > 1) {
+    const int kb_first = (wg_lo / 32) * 32, all_rounds = ((wg_last - kb_first) / 32 + 2) / 2;
+    const int mine = min(split.pieces, (all_rounds + split.piece_rounds - 1) / split.piece_rounds);  // pieces of this item
+    if (piece == 0 && threadIdx.x == 0) split.cut[item] = mine;
+    if (piece >= mine) return;
+    if (mine > 1) {
+      partial = true;
+      const int from = kb_first + 64 * split.piece_rounds * piece;  // the piece's first key
+      if (piece + 1 < mine) wg_last = from + 64 * split.piece_rounds - 1;
+      if (piece > 0) wg_lo = from;
+    }
+  }
 
   // this wave's queries
   const int unit = bz * 4 + wave;
@@ -965,6 +1001,18 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     }
   }
 
+  if (partial) {
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      if (!qok[qt]) continue;
+      const size_t at = ((size_t)(tok0 + q0 + qt * 16 + col) * H + head) * split.pieces + piece;
+      if (grp == 0) *reinterpret_cast<float2*>(split.ml + at * 2) = make_float2(m[qt], l[qt]);
+      float* arow = split.acc + at * D + 4 * grp;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(arow + dt * 16) = o[qt][dt];
+    }
+    return;
+  }
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     if (!qok[qt]) continue;
@@ -979,34 +1027,95 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   }
 }
 
+// The pieces of every cut item, put together: one workgroup per item, its waves and lanes holding the queries and
+// coordinates they hold in the kernel above.  out = sum_j acc_j 2^(m_j - m) / sum_j l_j 2^(m_j - m) with m the
+// largest maximum; a piece that saw no key has m = -inf and l = 0.
+template <int DC, int QT>
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const int* __restrict__ tiles, bf16* __restrict__ out,
+                                                                  int H, int KV, int units_z, PrefillSplit split) {
+  constexpr int D = DC * 32, DT = DC * 2, WQ = 16 * QT, PARTS = 64 / WQ;
+  const int item = blockIdx.x;
+  const int n = split.cut[item];
+  if (n <= 1) return;
+  const int G = H / KV, per_tile = KV * units_z;
+  const int tile = item / per_tile, kvh = (item % per_tile) / units_z, bz = item % units_z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
+  const int tok0 = tiles[4 * tile], count = tiles[4 * tile + 1];
+  const int unit = bz * 4 + wave, head = kvh * G + unit % G, q0 = (unit / G) * WQ;
+  if (unit >= PARTS * G || q0 >= count) return;
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int qi = q0 + qt * 16 + col;
+    if (qi >= count) continue;
+    const size_t at = ((size_t)(tok0 + qi) * H + head) * split.pieces;
+    const float2* ml = reinterpret_cast<const float2*>(split.ml) + at;  // (m, l) of the pieces
+    float m = NEG_INF;
+    for (int j = 0; j < n; ++j) m = fmaxf(m, ml[j].x);
+    f32x4_t sum[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) sum[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    for (int j = 0; j < n; ++j) {
+      const float2 p = ml[j];
+      const float w = p.x == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(p.x - m);
+      den += p.y * w;
+      const float* a = split.acc + (at + j) * D + 4 * grp;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) sum[dt] += *reinterpret_cast<const f32x4_t*>(a + dt * 16) * w;
+    }
+    const float inv = 1.0f / den;
+    bf16* orow = out + ((size_t)(tok0 + qi) * H + head) * D + 4 * grp;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const bf16x4_t r4 = {(bf16)(sum[dt][0] * inv), (bf16)(sum[dt][1] * inv), (bf16)(sum[dt][2] * inv), (bf16)(sum[dt][3] * inv)};
+      *reinterpret_cast<bf16x4_t*>(orow + dt * 16) = r4;
+    }
+  }
+}
+
 // tiles: [num_tiles, 4] int32 (first flat token, count <= 64, block-table row, first position);
 // fastest when sorted by first position + count, largest first.
 // query_tiles: 2, a wave owns 32 queries of a head and a workgroup two heads' 64; or 1, a wave owns 16 and a
 // workgroup one head's 64: twice the workgroups, each with half the arithmetic for the same keys and values
 // brought into LDS, so that a round of 64 keys is shorter.  That pays where few work items decide the time
 // (a lone prompt of a few thousand tokens: its last tile's rounds are a chain that nothing shortens).
+// pieces > 1: every work item comes as that many workgroups, and items of more than piece_rounds rounds of 64 keys are
+// cut along their keys into pieces of that many rounds and merged by a second kernel (see PrefillSplit); the caller
+// then brings cut [num_tiles * KV * units] int32 with units = ceil(64 / (16 query_tiles) * (H / KV) / 4), part_ml
+// [T, H, pieces, 2] and part_acc [T, H, pieces, D] fp32, T being one more than the largest flat token of a tile, and
+// piece_rounds * pieces covers the longest item.  pieces <= 1: none is cut, the three may be null.
 extern "C" int as_attn_prefill_mfma(const void* q, const void* k_pages, const void* v_pages, const int* tiles,
                                     int num_tiles, const int* block_tables, int table_width, void* out, int H,
                                     int KV, int D, int bs, float scale, int window, int query_tiles,
+                                    int pieces, int piece_rounds, int* cut, float* part_ml, float* part_acc,
                                     hipStream_t stream) {
   if (num_tiles <= 0) return AS_OK;
   if (H <= 0 || KV <= 0 || H % KV || bs <= 0 || table_width <= 0) return AS_BAD_SHAPE;
   const int G = H / KV;
   if (D % 32 || D <= 0 || D > 256 || bs % 16) return AS_BAD_SHAPE;
   if (query_tiles != 1 && query_tiles != 2) return AS_BAD_SHAPE;
+  if (pieces < 1) pieces = 1;
+  if (pieces > 1 && (piece_rounds < PREFILL_MIN_PIECE_ROUNDS || !cut || !part_ml || !part_acc)) return AS_BAD_SHAPE;
   const int units_z = (64 / (16 * query_tiles) * G + 3) / 4;
   const long items = (long)num_tiles * KV * units_z;
-  if (items > 0x7fffffffL) return AS_BAD_SHAPE;
+  const long blocks = items * pieces;
+  if (blocks > 0x7fffffffL) return AS_BAD_SHAPE;
   const int pass = compute_units();
+  const PrefillSplit split{pieces, piece_rounds, cut, part_ml, part_acc};
 #define LAUNCH(DCV)                                                                                   \
-  if (query_tiles == 1)                                                                               \
-    attn_prefill_mfma_kernel<DCV, 1><<<(int)items, 256, 0, stream>>>(                                 \
+  if (query_tiles == 1) {                                                                             \
+    attn_prefill_mfma_kernel<DCV, 1><<<(int)blocks, 256, 0, stream>>>(                                \
         (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, tiles, block_tables, table_width, \
-        (bf16*)out, H, KV, bs, scale, window, units_z, pass);                                         \
-  else                                                                                                \
-  attn_prefill_mfma_kernel<DCV, 2><<<(int)items, 256, 0, stream>>>(                                   \
-      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, tiles, block_tables, table_width,   \
-      (bf16*)out, H, KV, bs, scale, window, units_z, pass)
+        (bf16*)out, H, KV, bs, scale, window, units_z, pass, split);                                  \
+    if (pieces > 1)                                                                                   \
+      attn_prefill_merge_kernel<DCV, 1><<<(int)items, 256, 0, stream>>>(tiles, (bf16*)out, H, KV, units_z, split); \
+  } else {                                                                                            \
+    attn_prefill_mfma_kernel<DCV, 2><<<(int)blocks, 256, 0, stream>>>(                                \
+        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, tiles, block_tables, table_width, \
+        (bf16*)out, H, KV, bs, scale, window, units_z, pass, split);                                  \
+    if (pieces > 1)                                                                                   \
+      attn_prefill_merge_kernel<DCV, 2><<<(int)items, 256, 0, stream>>>(tiles, (bf16*)out, H, KV, units_z, split); \
+  }
   switch (D / 32) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;

@@ -27,7 +27,7 @@ SIGNATURES = {
     "as_attn_single_query": ("attention", [P, P, P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
     "as_attn_decode_mfma": ("attention", [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
     "as_attn_decode_fresh": ("attention", [P, P, P, I, P, P, F, I, P, P, P, I, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
-    "as_attn_prefill_mfma": ("attention", [P, P, P, P, I, P, I, P, I, I, I, I, F, I, I, P]),
+    "as_attn_prefill_mfma": ("attention", [P, P, P, P, I, P, I, P, I, I, I, I, F, I, I, I, I, P, P, P, P]),
     "as_gemm_f32": ("gemm", [P, P, P, I, I, I, P]),
     "as_gemm_bf16_skinny": ("gemm", [P, P, P, P, I, I, I, I, I, P]),
     "as_gemm_bf16_gated": ("gemm", [P, P, P, P, I, I, I, P]),

@@ -395,6 +395,32 @@ def _prefill_query_tiles(num_tiles: int, H: int, KV: int) -> int:
 
 
 
+# A step of few work items lasts as long as its longest: a portion of 512 tokens behind 3,584 cached ones is 128
+# workgroups of 57 to 64 rounds of 64 keys on a GPU with places for 512.  Where the places allow, every item comes as
+# several workgroups, and the items of more rounds than a piece has are cut along their keys into such pieces, merged
+# by a second kernel (csrc/attention.hip, PrefillSplit).  The merge costs some 10 us, and pieces that outnumber the
+# places wait for one: a lone prompt (items of 1 round up to all, as many as places at 2,048 tokens) is slower cut.
+PREFILL_PIECES = None  # a number to force that many pieces (1: none; measurements and tests); None: by the sizes
+PREFILL_MAX_PIECES = 8
+PREFILL_MIN_PIECE_ROUNDS = 8  # a piece has at least this many rounds ...
+PREFILL_MIN_ROUNDS = 28  # ... and the longest item this many, or nothing is cut (at 24 the merge costs what the cut gains)
+
+
+def _prefill_pieces(num_tiles: int, H: int, KV: int, query_tiles: int, max_context: int, window: int = 0) -> tuple:
+    """(pieces, rounds of a piece) for a prompt step; (1, 0): nothing is cut."""
+    units = -(-(64 // (16 * query_tiles)) * (H // KV) // 4)
+    span = min(max_context, window + 64) if window > 0 else max_context  # the keys that the longest item walks
+    rounds = -(-span // 64)
+    if PREFILL_PIECES is not None:
+        pieces = max(1, min(int(PREFILL_PIECES), rounds // 2))
+    elif rounds < PREFILL_MIN_ROUNDS:
+        pieces = 1
+    else:
+        places = 2 * compute_units()
+        pieces = min(PREFILL_MAX_PIECES, places // (num_tiles * KV * units), rounds // PREFILL_MIN_PIECE_ROUNDS)
+    return (pieces, -(-rounds // pieces)) if pieces > 1 else (1, 0)
+
+
 def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context, query_tiles=None) -> None:
     """Causal attention of prompt portions over the paged cache, bfloat16, on the matrix cores.
 
@@ -418,9 +444,16 @@ def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, m
         raise KernelError("attention: block tables are shorter than the longest context")
     if query_tiles is None:
         query_tiles = PREFILL_QUERY_TILES or _prefill_query_tiles(tiles.shape[0], H, KV)
+    pieces, piece_rounds = _prefill_pieces(tiles.shape[0], H, KV, query_tiles, max_context, window)
+    cut = part_ml = part_acc = None
+    if pieces > 1:
+        units = -(-(64 // (16 * query_tiles)) * (H // KV) // 4)
+        cut = torch.empty(tiles.shape[0] * KV * units, dtype=I32, device=q.device)
+        part_ml = torch.empty((T, H, pieces, 2), dtype=F32, device=q.device)
+        part_acc = torch.empty((T, H, pieces, D), dtype=F32, device=q.device)
     call("as_attn_prefill_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(tiles), tiles.shape[0],
          _ptr(block_tables), block_tables.shape[1], _ptr(out), H, KV, D, bs, float(scale), int(window),
-         int(query_tiles), _stream())  # fmt: skip
+         int(query_tiles), pieces, piece_rounds, _ptr(cut), _ptr(part_ml), _ptr(part_acc), _stream())  # fmt: skip
 
 
 SKINNY_MAX_ROWS = 16  # up to here the bf16 product streams the weights through our own kernel

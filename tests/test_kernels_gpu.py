@@ -902,10 +902,11 @@ def test_attention_prefill(ops, H, KV, D, bs, window):
             tiles.append([flat + q0, min(64, n - q0), r, start + q0])
         flat += n
     ref = pk.paged_attention(q, k_pages, v_pages, i32(list(range(T))), i32(positions), i32(tok_row), tables, D**-0.5, window)
-    for query_tiles in (None, 1, 2):  # as the sizes choose; a wave owning 16 queries; 32
+    for query_tiles, cut in [(None, None), (1, 1), (2, 1), (1, 2), (2, 3), (2, 4)]:  # as the sizes choose; a wave owning 16 queries; 32; long items cut into pieces
         out = torch.zeros(T, H, D, dtype=BF16, device=DEV)
-        ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, window, max(lens), query_tiles=query_tiles)
-        assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), (query_tiles, (out.float() - ref).abs().max())
+        with prefill_cut(ops, cut):
+            ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, window, max(lens), query_tiles=query_tiles)
+        assert torch.allclose(out.float(), ref, atol=2e-2, rtol=2e-2), (query_tiles, cut, (out.float() - ref).abs().max())
 
 
 def test_attention_prefill_of_a_long_prompt_in_one_step(ops):
@@ -918,9 +919,10 @@ def test_attention_prefill_of_a_long_prompt_in_one_step(ops):
     tiles = sorted(([q0, min(64, n - q0), 0, start + q0] for q0 in range(0, n, 64)), key=lambda t: -(t[3] + t[1]))
     check = list(range(0, n, 97)) + [n - 1]
     ref = pk.paged_attention(q, k_pages, v_pages, i32(check), i32(list(range(start, start + n))), i32([0] * n), tables, D**-0.5)
-    for query_tiles in (2, 1):
+    for query_tiles, cut in ((2, 1), (1, 1), (2, 2), (1, 5)):
         out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
-        ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, 0, start + n, query_tiles=query_tiles)
+        with prefill_cut(ops, cut):
+            ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, D**-0.5, 0, start + n, query_tiles=query_tiles)
         assert torch.allclose(out[check].float(), ref[check], atol=2e-2, rtol=2e-2), (out[check].float() - ref[check]).abs().max()
 
 
@@ -934,10 +936,83 @@ def test_attention_prefill_sees_a_far_key_and_not_the_future(ops):
         fut_page, fut_off = int(tables[0, 651 // bs]), 651 % bs
         k_pages[fut_page, 0, fut_off] = (q[650, 0].float() * 8.0).to(BF16)  # a stronger match, one step in the future
         tiles = [[q0, min(64, n - q0), 0, q0] for q0 in range(0, n, 64)]
-        for query_tiles in (1, 2):
+        for query_tiles, cut in ((1, 1), (2, 1), (2, 2), (1, 3), (2, 5)):  # cut: the far key lies in one piece, the future one in the last
             out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
-            ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, 1.0, 0, n, query_tiles=query_tiles)
-            assert torch.allclose(out[650, 0].float(), v_pages[page, 0, :, off].float(), atol=2e-2), (far, query_tiles)
+            with prefill_cut(ops, cut):
+                ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, out, 1.0, 0, n, query_tiles=query_tiles)
+            assert torch.allclose(out[650, 0].float(), v_pages[page, 0, :, off].float(), atol=2e-2), (far, query_tiles, cut)
+
+
+class prefill_cut:
+    """Within it, `ops.attn_prefill` cuts long work items into that many pieces (1: never; None: as the sizes say)."""
+
+    def __init__(self, ops, pieces):
+        self.ops, self.pieces = ops, pieces
+
+    def __enter__(self):
+        self.before, self.ops.PREFILL_PIECES = self.ops.PREFILL_PIECES, self.pieces
+
+    def __exit__(self, *exc):
+        self.ops.PREFILL_PIECES = self.before
+
+
+@pytest.mark.parametrize("H,KV,D,bs,n,start,window,pieces", [
+    (32, 8, 128, 16, 2048, 0, 0, 2), (16, 8, 128, 16, 1000, 0, 0, 3), (6, 2, 32, 16, 777, 130, 0, 2), (8, 2, 64, 32, 1500, 0, 1000, 4),
+    (64, 8, 128, 16, 640, 64, 0, 2), (32, 8, 128, 16, 512, 3584, 0, 4), (32, 8, 128, 16, 200, 9000, 0, 8), (4, 4, 256, 16, 300, 2100, 0, 5)])
+def test_long_items_of_a_prompt_step_are_cut_into_pieces_and_merged(ops, H, KV, D, bs, n, start, window, pieces):
+    """A step of few work items lasts as long as the longest: items of more rounds than a piece has are cut along
+    their keys, the pieces' maxima, sums and outputs merged.  The entry point called as the wrapper calls it, on a
+    lone prompt (items of every length: some are cut, in two or more, and some are not) and on a portion behind a
+    long prefix (all are): the result is the plain attention's, and the kernel's without the cut."""
+    from atomserve_amd.kernels.lib import call
+
+    torch.manual_seed(n + H)
+    _, k_pages, v_pages, tables, _ = paged_case(BF16, H, KV, D, bs, [start + n], seed=4, k_scale=2.0 / math.sqrt(D / 16))
+    q = torch.randn(n, H, D, device=DEV).to(BF16)
+    tiles = sorted(([q0, min(64, n - q0), 0, start + q0] for q0 in range(0, n, 64)), key=lambda t: -(t[3] + t[1]))
+    check = sorted({0, 1, min(63, n - 1), min(64, n - 1), n // 2 - 1, n // 2, min(n - 1, n // 2 + 70), max(0, n - 65), n - 2, n - 1} | set(range(5, n, 211)))
+    ref = pk.paged_attention(q, k_pages, v_pages, i32(check), i32(list(range(start, start + n))), i32([0] * n), tables, D**-0.5, window)
+    stream = torch.cuda.current_stream().cuda_stream
+    for query_tiles in (2, 1):
+        with prefill_cut(ops, pieces):
+            got_pieces, piece_rounds = ops._prefill_pieces(len(tiles), H, KV, query_tiles, start + n, window)
+        span = min(start + n, window + 64) if window else start + n
+        assert got_pieces == pieces and piece_rounds == -(-(-(-span // 64)) // pieces)
+        units = -(-(64 // (16 * query_tiles)) * (H // KV) // 4)
+        cut = torch.full((len(tiles) * KV * units,), -1, dtype=I32, device=DEV)
+        part_ml = torch.full((n, H, pieces, 2), float("nan"), device=DEV)
+        part_acc = torch.full((n, H, pieces, D), float("nan"), device=DEV)
+        out = torch.zeros(n, H, D, dtype=BF16, device=DEV)
+        call("as_attn_prefill_mfma", q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), i32(tiles).data_ptr(), len(tiles),
+             tables.data_ptr(), tables.shape[1], out.data_ptr(), H, KV, D, bs, D**-0.5, window, query_tiles, pieces, piece_rounds,
+             cut.data_ptr(), part_ml.data_ptr(), part_acc.data_ptr(), stream)  # fmt: skip
+        said = set(cut.tolist())
+        assert said <= set(range(1, pieces + 1)) and pieces in said  # every item said how many pieces it is; the longest all of them
+        # (a work item is a tile's queries of some heads: those of a tile may be cut differently, and a tile of fewer
+        # than 64 queries leaves some of its workgroups without work)
+        full = [i for i, t in enumerate(tiles) if t[1] == 64]
+        per_tile = cut.view(len(tiles), -1).float().mean(1)[full]
+        assert bool((per_tile[:-1] >= per_tile[1:]).all())  # the more keys an item sees, the more pieces
+        if start == 0:
+            assert 1 in said and per_tile[-1] == 1  # the first tile of a lone prompt is not cut
+        assert torch.allclose(out[check].float(), ref[check], atol=2e-2, rtol=2e-2), (out[check].float() - ref[check]).abs().max()
+        whole = torch.zeros(n, H, D, dtype=BF16, device=DEV)
+        with prefill_cut(ops, 1):
+            ops.attn_prefill(q, k_pages, v_pages, i32(tiles), tables, whole, D**-0.5, window, start + n, query_tiles=query_tiles)
+        assert torch.allclose(out.float(), whole.float(), atol=2e-2, rtol=2e-2)  # every token, against the kernel without the cut
+
+
+def test_what_the_sizes_say_about_cutting_prompt_steps(ops):
+    """A portion behind a long prefix is few long items: cut, into as many pieces as fill the GPU's places, of at least
+    eight rounds each.  A lone prompt, a short context, or as many items as places: not cut."""
+    cus = ops.compute_units()
+    tiles_of = lambda tokens: -(-tokens // 64)
+    assert ops._prefill_pieces(tiles_of(512), 32, 8, 2, 4096) == (min(4, 2 * cus // 128), -(-64 // min(4, 2 * cus // 128)))
+    assert ops._prefill_pieces(tiles_of(512), 32, 8, 2, 2048)[0] == min(4, 2 * cus // 128)
+    assert ops._prefill_pieces(tiles_of(64), 32, 8, 2, 20000)[0] == min(8, 2 * cus // 16)
+    assert ops._prefill_pieces(tiles_of(2048), 32, 8, 2, 2048) == (1, 0) or cus > 256  # a lone prompt: as many items as places
+    assert ops._prefill_pieces(tiles_of(512), 32, 8, 2, 1024) == (1, 0)  # 16 rounds: too short to pay for the merge
+    assert ops._prefill_pieces(tiles_of(512), 32, 8, 2, 8192, window=512) == (1, 0)  # a window keeps every item short
 
 
 def test_kernels_refuse_what_they_cannot_do(ops):

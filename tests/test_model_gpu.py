@@ -739,3 +739,35 @@ def test_a_replay_step_that_cannot_run_changes_nothing(setup):
     for got, place in ((first[0], 19), (rest[0], 39)):
         assert float((got - ref[place]).abs().max()) <= rc.TOL_FLOAT32 * max(1.0, float(ref.abs().max()))
     assert replay.manager.num_free == replay.manager.num_blocks and not replay.live
+
+
+def test_portions_behind_a_long_prefix_cut_their_attention(tmp_path, monkeypatch):
+    """Portions of a prompt behind some two thousand cached tokens are few work items of many rounds of keys: the
+    prefill attention cuts them along their keys and merges the pieces.  Through the step function, beside another
+    request's portion and decoded tokens: every row is the plain model's, within what rounding alone does."""
+    from atomserve_amd.kernels import ops
+
+    raw = dict(TINY["B"], max_position_embeddings=4096)
+    weights = plain_random_weights(raw, seed=53, std=0.2, gain_std=0.2)
+    path = write_model_dir(str(tmp_path / "long"), raw, weights, torch.bfloat16)
+    vocab = raw["vocab_size"]
+    requests = {"a": rc.random_ids(vocab, 2400, seed=8), "b": rc.random_ids(vocab, 300, seed=9)}
+    a, b = requests["a"], requests["b"]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:1900], "want": [0, 1899]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[1900:2030], "want": list(range(0, 130, 9))}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[2030:2094], "want": [0, 63]}, {"id": "b", "tokens": b[:200], "want": [199]}], "end": []},
+        {"step": 3, "entries": [{"id": "b", "tokens": [b[200]], "want": [0]}, {"id": "a", "tokens": a[2094:2294], "want": list(range(0, 200, 7))}], "end": []},
+        {"step": 4, "entries": [{"id": "a", "tokens": a[2294:2303], "want": [8]}, {"id": "b", "tokens": b[201:300], "want": [98]}], "end": ["b"]},
+        {"step": 5, "entries": [{"id": "a", "tokens": a[2303:], "want": [0, 96]}], "end": ["a"]},
+    ]
+    decided = []
+    real = ops._prefill_pieces
+    monkeypatch.setattr(ops, "_prefill_pieces", lambda *args, **kw: decided.append(real(*args, **kw)) or decided[-1])
+    replay = make_replay(path, "bfloat16", rc.live_token_bound(steps))
+    result = compare(replay, steps, requests, raw, weights, {}, "bfloat16", plain_kwargs={"batched": True})
+    assert result.rows == 2 + 15 + 3 + 30 + 2 + 2
+    # every step's attention had its pieces decided, layer by layer; with so few heads even the lone first portion is cut
+    assert len(decided) == len(steps) * raw["num_hidden_layers"] and all(pieces > 1 for pieces, _ in decided[3:])
+    assert len({pieces for pieces, _ in decided}) > 1  # into more pieces where the items are fewer
+    assert replay.manager.num_free == replay.manager.num_blocks
