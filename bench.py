@@ -64,7 +64,9 @@ def parse_args():
     p.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt whose prefill is timed "
-                   "(longer than 2,048: in steps of 2,048 tokens)")  # fmt: skip
+                   "(longer than the step budget: in portions of it)")  # fmt: skip
+    p.add_argument("--budget", type=int, default=None, help="token budget of a step (default: 2,048, or --context if that "
+                   "is more): prompts longer than this are prefilled in portions of it")  # fmt: skip
     p.add_argument("--no-calibration", action="store_true", help="skip the library copy and matmul probes")
     p.add_argument("--greedy", action="store_true", help="greedy instead of the default sampling settings")
     p.add_argument("--workload", choices=["decode", "mixed"], default="decode",
@@ -209,11 +211,11 @@ def main() -> int:
     block = args.block_size
     max_len = max(args.max_len, args.context + args.steps + args.warmup + 16 + (64 if args.profile else 0),
                   args.prefill_tokens + 16)
-    num_blocks = max(batches) * max_len // block
+    num_blocks = max(batches) * -(-max_len // block)
     params = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True) if args.greedy else \
         SamplingParams(max_tokens=100000, ignore_eos=True)  # fmt: skip
     engine_config = EngineConfig(block_size=block, num_blocks=num_blocks, max_num_seqs=max(batches),
-                                 max_num_batched_tokens=max(2048, args.context), max_model_len=max_len,
+                                 max_num_batched_tokens=args.budget or max(2048, args.context), max_model_len=max_len,
                                  enable_prefix_caching=False)  # fmt: skip
     engine = create_engine(model, engine_config, seed=0)
     engine.warm_up()  # as the command line does before it serves: decode steps captured, prompt lengths tried
@@ -310,7 +312,8 @@ def main() -> int:
             "model": f"Qwen3-{args.sizes.upper()} sizes", "layers": c.num_layers, "layers_full": full_layers, "hidden": c.hidden_size,
             "heads": c.num_heads, "kv_heads": c.num_kv_heads, "head_dim": c.head_dim,
             "intermediate": c.intermediate_size, "vocab": c.vocab_size, "global_batch": args.batch,
-            "seq_len": args.context, "shortest_context": args.shortest_context or args.context, "max_context": max_len, "block_size": block, "parallelism": "single GPU",
+            "seq_len": args.context, "shortest_context": args.shortest_context or args.context, "max_context": max_len, "block_size": block,
+            "step_budget": engine_config.max_num_batched_tokens, "parallelism": "single GPU",
             "sampling": "greedy" if args.greedy else "temperature 0.6 top-k 20 top-p 0.95",
         },
         "roofline": roofline(args.batch, mean_ctx, ms),
