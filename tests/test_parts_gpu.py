@@ -2,7 +2,8 @@
 that are not Qwen3, registered from here without a change to the package: a mixer with a
 fixed-size state of its own in some layers, a feed-forward that routes each token to one of
 several experts, a position encoding that turns half of each head by slowed positions, a layer
-that runs twice, and a run that reads the cache another run wrote."""
+that runs twice, a run that reads the cache another run wrote, a mixer that keeps nothing and sorts
+a step's rows its own way, another norm and another arrangement of a layer."""
 
 import dataclasses
 import math
@@ -861,3 +862,135 @@ def test_mixers_that_sort_the_rows_differently_share_a_step(dtype):
     for rc, _ in caches.values():
         engine.scheduler.manager.release(rc)
     assert engine.scheduler.manager.num_free == engine.scheduler.manager.num_blocks
+
+
+# ---- another norm and another arrangement of a layer, defined here ---------------------------------
+
+
+def make_centred_norm():
+    from atomserve_amd.parts.base import Norm, SplitSums, WeightDecl
+
+    class CentredNorm(Norm):
+        """weight * (x - mean(x)) / sqrt(var(x) + eps): a norm that is not the package's, computed with library
+        calls on the fp32 stream.  Like every norm it first adds the pending output of the part before."""
+
+        def weight_decls(self):
+            return {"weight": WeightDecl((self.spec.size,), role="vector")}
+
+        def forward(self, x, delta=None, rows=None, update_residual=True):
+            assert not isinstance(delta, SplitSums)  # it does not say `takes_split_sums`, so nobody hands it any
+            v = x if delta is None else x + delta.float()
+            if delta is not None and update_residual:
+                x.copy_(v)
+            if rows is not None:
+                v = v[rows.long()]
+            centred = v - v.mean(-1, keepdim=True)
+            out = centred / torch.sqrt(centred.pow(2).mean(-1, keepdim=True) + self.spec.eps) * self.weight.float()
+            return out.to(self.env.dtype)
+
+    return CentredNorm
+
+
+def make_parallel_block():
+    from atomserve_amd.parts.base import Arrangement, build
+
+    class ParallelBlock(Arrangement):
+        """x += mixer(norm(x)) + ffn(norm(x)): one norm feeds both parts, and their outputs are added together
+        before they join the stream (in the next norm, as a pending sum)."""
+
+        def __init__(self, spec, env):
+            super().__init__(spec, env)
+            self.norm = build("norm", spec.mixer_norm, env)
+            self.mixer = build("mixer", spec.mixer, env)
+            self.ffn = build("feed_forward", spec.ffn, env)
+
+        def parts(self):
+            return {"mixer_norm": self.norm, "mixer": self.mixer, "ffn": self.ffn}
+
+        def forward(self, x, delta, step, cache, next_norm=None):
+            h = self.norm.forward(x, delta)
+            mixed = self.mixer.forward(h, step, cache)
+            fed = self.ffn.forward(h, step)
+            return (mixed.float() + fed.float()).to(self.env.dtype)
+
+    return ParallelBlock
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_another_norm_and_another_arrangement_of_a_layer(dtype):
+    """Every norm of the model is a centred one defined here, and every layer adds its mixer and its feed-forward
+    side by side from one norm instead of one after the other: registered from here, built by the plan, loaded by
+    name (the second norm's gains are not in the checkpoint and not asked for), stepped whole, in portions and token
+    by token beside another request."""
+    from atomserve_amd.config.registry import Architecture, architecture_for, register_architecture
+    from atomserve_amd.parts.base import register
+
+    register("norm", "toy_centred", make_centred_norm(), replace=True)
+    register("arrangement", "toy_parallel", make_parallel_block(), replace=True)
+    qwen = architecture_for(TINY_B)
+
+    def build_plan(c):
+        plan = qwen.build_plan(c)
+        centred = lambda spec: dataclasses.replace(spec, kind="toy_centred")
+        layers = tuple(dataclasses.replace(layer, arrangement="toy_parallel", mixer_norm=centred(layer.mixer_norm),
+                                           ffn_norm=centred(layer.ffn_norm)) for layer in plan.layers)  # fmt: skip
+        return dataclasses.replace(plan, layers=layers, final_norm=centred(plan.final_norm))
+
+    def checkpoint_map(c):
+        return {k: v for k, v in qwen.checkpoint_map(c).items() if ".ffn_norm." not in k}
+
+    def checkpoint_shapes(c):
+        return {k: v for k, v in qwen.checkpoint_shapes(c).items() if "post_attention_layernorm" not in k}
+
+    arch = register_architecture(
+        Architecture("ParallelCentredForCausalLM", qwen.parse_config, build_plan, checkpoint_map, checkpoint_shapes), replace=True
+    )
+    raw = {**TINY_B, "architectures": ["ParallelCentredForCausalLM"], "num_hidden_layers": 3}
+    w = {k: v for k, v in plain_random_weights(raw, seed=14, std=0.2, gain_std=0.2).items() if "post_attention_layernorm" not in k}
+    engine = build_engine(arch, raw, w, dtype)
+    assert not engine.runner.model.capturable  # the norm defined here does not say it may be captured: steps run one by one
+
+    def centred(x, weight, eps):
+        c = x - x.mean(-1, keepdim=True)
+        return c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * weight
+
+    def reference(ids):
+        cfg = plain.normalise_config(raw)
+        wd = {k: v.double() for k, v in w.items()}
+        pos = torch.arange(len(ids))
+        x = plain.embed(wd["model.embed_tokens.weight"], torch.as_tensor(ids))
+        for i in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{i}."
+            h = centred(x, wd[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+            fed = plain.swiglu(h, wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"], wd[p + "mlp.down_proj.weight"])
+            x = x + plain.attention_layer(h, wd, p, cfg, pos) + fed
+        x = centred(x, wd["model.norm.weight"], cfg["rms_norm_eps"])
+        return (x @ wd["lm_head.weight"].T).float()
+
+    a = torch.randint(0, 1000, (75,), generator=torch.Generator().manual_seed(31)).tolist()
+    b = torch.randint(0, 1000, (20,), generator=torch.Generator().manual_seed(32)).tolist()
+    ref = {"a": reference(a), "b": reference(b)}
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    caches = {}
+    whole = step_rows(engine, caches, [("whole", a, list(range(75)))])
+    assert (whole - ref["a"]).abs().max() <= tol * max(1.0, ref["a"].abs().max())
+    got = {"a": [], "b": []}
+    logits = step_rows(engine, caches, [("a", a[:66], list(range(66))), ("b", b[:2], [0, 1])])
+    got["a"].append(logits[:66]); got["b"].append(logits[66:])  # noqa: E702
+    for i in range(9):
+        logits = step_rows(engine, caches, [("b", b[2 + 2 * i : 4 + 2 * i], [0, 1]), ("a", [a[66 + i]], [0])])
+        got["b"].append(logits[:2]); got["a"].append(logits[2:])  # noqa: E702
+    for name in "ab":
+        assert (torch.cat(got[name]) - ref[name]).abs().max() <= tol * max(1.0, ref[name].abs().max()), name
+    for rc, _ in caches.values():
+        engine.scheduler.manager.release(rc)
+    assert engine.scheduler.manager.num_free == engine.scheduler.manager.num_blocks
+    # and through the scheduler: greedy generation equals the plain model's
+    if dtype == torch.float32:
+        from atomserve_amd.engine.sequence import SamplingParams
+
+        out = engine.generate([a[:9]], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0]
+        seq = list(a[:9])
+        for t in out:
+            assert t == int(reference(seq)[-1].argmax())
+            seq.append(t)
