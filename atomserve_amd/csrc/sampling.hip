@@ -315,6 +315,51 @@ extern "C" int as_apply_penalty(float* logits, const int* rows, const int* cols,
 }
 
 // ---- the full pipeline ------------------------------------------------------------
+// The draw among a row's candidates, ranked best first in sel[0..found-1] (found <= blockDim.x): softmax at
+// temperature T over them, the best ones kept while the mass ranked above is below p_keep, and the
+// exponential race among those.  Block-wide, every thread calls it; thread 0 returns the choice's place in
+// `sel` (0 for fewer than two candidates), the others nothing of use.  The exponentials, the noise and the
+// quotients are one candidate per thread; the two sums run over them in order in one thread, so the
+// result is that of the plain loop over the candidates, whatever the block's size.
+// work: __shared__ float[3 * (most candidates) + 1].
+__device__ __forceinline__ int draw_among_ranked(const unsigned long long* sel, int found, float T, float p_keep,
+                                                 long long seed, int counter, float* work) {
+  if (found <= 1) return 0;  // uniform over the block
+  const int tid = threadIdx.x;
+  float* e = work;
+  float* noise = work + found;
+  float* score = work + 2 * found;
+  float* total = work + 3 * found;
+  const float v0 = key_value(sel[0]);
+  if (tid < found) {
+    e[tid] = expf((key_value(sel[tid]) - v0) / T);
+    noise[tid] = exp1_noise(seed, counter, tid);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float sum = 0.f;
+    for (int i = 0; i < found; ++i) sum += e[i];
+    *total = sum;
+  }
+  __syncthreads();
+  if (tid < found) {
+    const float p = e[tid] / *total;
+    e[tid] = p;
+    score[tid] = p / noise[tid];
+  }
+  __syncthreads();
+  int choice = 0;
+  if (tid == 0) {
+    float mass = 0.f, best_score = -1.f;
+    for (int i = 0; i < found; ++i) {
+      if (mass >= p_keep) break;  // the mass ranked above already reaches top_p
+      mass += e[i];
+      if (score[i] > best_score) { best_score = score[i]; choice = i; }
+    }
+  }
+  return choice;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const long long* __restrict__ seeds, const int* __restrict__ counters,
@@ -323,7 +368,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   unsigned long long* red = topk_shared.red;
   __shared__ float fred[17];
   __shared__ unsigned long long sel[SAMPLE_KMAX];
-  __shared__ float ework[SAMPLE_KMAX];
+  __shared__ float ework[3 * SAMPLE_KMAX + 1];
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* x = logits + (size_t)row * V;
   float T = temperature[row];
@@ -338,27 +383,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (!all && !wide) {
     const int found = block_topk(x, V, k, sel, topk_shared);
     __syncthreads();
-    if (tid == 0) {
-      int choice = 0;
-      if (found > 1) {
-        const float v0 = key_value(sel[0]);
-        float sum = 0.f;
-        for (int i = 0; i < found; ++i) {
-          const float e = expf((key_value(sel[i]) - v0) / T);
-          ework[i] = e;
-          sum += e;
-        }
-        float mass = 0.f, best_score = -1.f;
-        for (int i = 0; i < found; ++i) {
-          const float p = ework[i] / sum;
-          if (mass >= p_keep) break;  // the mass ranked above already reaches top_p
-          mass += p;
-          const float score = p / exp1_noise(seed, counter, i);
-          if (score > best_score) { best_score = score; choice = i; }
-        }
-      }
-      out[row] = found ? key_index(sel[choice]) : 0;
-    }
+    const int choice = draw_among_ranked(sel, found, T, p_keep, seed, counter, ework);
+    if (tid == 0) out[row] = found ? key_index(sel[choice]) : 0;
     return;
   }
 
@@ -452,7 +478,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_candidates_kernel(
   __shared__ unsigned long long pool[SPLIT_SLICES * SPLIT_KMAX];
   __shared__ int first[SPLIT_SLICES + 1];
   __shared__ unsigned long long sel[SPLIT_KMAX];
-  __shared__ float ework[SPLIT_KMAX];
+  __shared__ float ework[3 * SPLIT_KMAX + 1];
   const int row = blockIdx.x, tid = threadIdx.x;
   float T = temperature[row];
   const float p_keep = top_p[row];
@@ -481,30 +507,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_candidates_kernel(
     if (rank < k) sel[rank] = key;
   }
   __syncthreads();
-  if (tid == 0) {
-    const int found = total < k ? total : k;
-    const long long seed = seeds[row];
-    const int counter = counters[row];
-    int choice = 0;
-    if (found > 1) {
-      const float v0 = key_value(sel[0]);
-      float sum = 0.f;
-      for (int i = 0; i < found; ++i) {
-        const float e = expf((key_value(sel[i]) - v0) / T);
-        ework[i] = e;
-        sum += e;
-      }
-      float mass = 0.f, best_score = -1.f;
-      for (int i = 0; i < found; ++i) {
-        const float p = ework[i] / sum;
-        if (mass >= p_keep) break;  // the mass ranked above already reaches top_p
-        mass += p;
-        const float score = p / exp1_noise(seed, counter, i);
-        if (score > best_score) { best_score = score; choice = i; }
-      }
-    }
-    out[row] = found ? key_index(sel[choice]) : 0;
-  }
+  const int found = total < k ? total : k;
+  const int choice = draw_among_ranked(sel, found, T, p_keep, seeds[row], counters[row], ework);
+  if (tid == 0) out[row] = found ? key_index(sel[choice]) : 0;
 }
 
 // As as_sample, for batches whose every row keeps between 1 and 64 candidates (greedy rows
