@@ -172,18 +172,22 @@ def main(argv=None) -> int:
     if not os.path.isfile(config_path):
         print(f"atomserve: no config.json at {config_path}", file=sys.stderr)
         return 1
-    with open(config_path) as f:
-        raw = json.load(f)
-    arch = architecture_for(raw)
-    config = arch.parse_config(raw)
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
-    print(f"Loading {args.model} ({args.dtype}, {arch.name}) ...", file=sys.stderr, flush=True)
-    model = DecoderModel(arch.build_plan(config), dtype, "cuda:0", stream_copies=not args.no_stream_copies)
-    if args.random_weights is not None:
-        source = DictSource(random_checkpoint(arch, config, args.random_weights, dtype=dtype, device="cuda:0"))
-        bind_checkpoint(model, arch, config, source, where="(random)")
-    else:
-        load_weights(model_dir, model, arch, config)
+    try:  # what is wrong with the folder is a message, not a traceback
+        with open(config_path) as f:
+            raw = json.load(f)
+        arch = architecture_for(raw)
+        config = arch.parse_config(raw)
+        print(f"Loading {args.model} ({args.dtype}, {arch.name}) ...", file=sys.stderr, flush=True)
+        model = DecoderModel(arch.build_plan(config), dtype, "cuda:0", stream_copies=not args.no_stream_copies)
+        if args.random_weights is not None:
+            source = DictSource(random_checkpoint(arch, config, args.random_weights, dtype=dtype, device="cuda:0"))
+            bind_checkpoint(model, arch, config, source, where="(random)")
+        else:
+            load_weights(model_dir, model, arch, config)
+    except (FileNotFoundError, ValueError) as error:  # a missing file, a config or a checkpoint that does not fit
+        print(f"atomserve: {error}", file=sys.stderr)
+        return 1
     block_bytes = CachePools.bytes_per_block(model.cache_requests(), args.block_size, dtype) or 1
     torch.cuda.synchronize()
     torch.cuda.empty_cache()  # what loading used for conversions counts as free

@@ -11,6 +11,7 @@ gains keep 32-bit storage when the checkpoint stores them so; integer tables int
 """
 
 import glob
+import json
 import os
 from contextlib import ExitStack
 from dataclasses import dataclass
@@ -112,12 +113,27 @@ class DictSource:
         return self.tensors[name]
 
 
+def missing_shards(model_dir: str) -> list:
+    """The weight files that a folder's index (model.safetensors.index.json, if it has one) names and the
+    folder does not hold: a partly copied or partly downloaded checkpoint is reported by its files, before
+    any tensor is looked for (reference atomserve/loader.py:28-40)."""
+    index = os.path.join(model_dir, "model.safetensors.index.json")
+    if not os.path.isfile(index):
+        return []
+    with open(index) as f:
+        named = set(json.load(f).get("weight_map", {}).values())
+    return sorted(name for name in named if not os.path.isfile(os.path.join(model_dir, name)))
+
+
 class SafetensorsSource:
     """Every *.safetensors file of a folder, memory-mapped; tensors are read one at a time."""
 
     def __init__(self, model_dir: str, stack: ExitStack):
         from safetensors import safe_open
 
+        absent = missing_shards(model_dir)
+        if absent:
+            raise FileNotFoundError(f"{model_dir} lacks {', '.join(absent)}, which its model.safetensors.index.json names")
         shards = sorted(glob.glob(os.path.join(model_dir, "*.safetensors")))
         if not shards:
             raise FileNotFoundError(f"no *.safetensors files in {model_dir}")

@@ -607,6 +607,33 @@ def test_command_line_generates(setup, capsys):
     assert runs[0] == runs[1] and len(runs[0]) == 6
 
 
+def test_command_line_says_what_a_folder_lacks(setup, tmp_path, capsys):
+    """A folder that cannot be served ends the command with a line that says why, not with a traceback: a
+    shard that the index names and the folder lacks (reference atomserve/loader.py:28-40), tensors of the
+    wrong shape, a config.json of another architecture."""
+    import json as js
+    import shutil
+
+    from atomserve_amd.engine.cli import main
+
+    name, raw, weights, path, _ = setup
+    tail = ["--prompt-ids", "1 2", "--kv-mem-gb", "0.01"]
+    partial = str(tmp_path / "partial")
+    shutil.copytree(path, partial)
+    with open(os.path.join(partial, "model.safetensors.index.json"), "w") as f:
+        js.dump({"weight_map": {k: ("model.safetensors" if i % 2 else "model-00002-of-00002.safetensors")
+                                for i, k in enumerate(sorted(weights))}}, f)  # fmt: skip
+    assert main([partial, *tail]) == 1
+    assert "lacks model-00002-of-00002.safetensors" in capsys.readouterr().err
+    wider = write_model_dir(str(tmp_path / "wider"), dict(raw, intermediate_size=raw["intermediate_size"] + 16), weights)
+    assert main([wider, *tail]) == 1
+    err = capsys.readouterr().err
+    assert "atomserve:" in err and "mlp.gate_proj.weight" in err and "Traceback" not in err
+    other = write_model_dir(str(tmp_path / "other"), dict(raw, architectures=["SomethingElseForCausalLM"]), weights)
+    assert main([other, *tail]) == 1
+    assert "SomethingElseForCausalLM" in capsys.readouterr().err
+
+
 def test_engine_thread_under_concurrent_clients(setup):
     """Two seconds of serving on the engine's own thread: clients on eight threads submit prompts
     of all lengths (some share a prefix), stream, and abort now and then, with a pool small

@@ -1,6 +1,7 @@
 """Weights by tensor name, their storage, the one error that lists everything wrong, and
 the random-weights folder (reference atomserve/loader.py:63-148)."""
 
+import json
 import os
 
 import pytest
@@ -112,6 +113,15 @@ def test_sharded_folder_is_read_across_files(tmp_path):
     save_file({k: w[k].bfloat16() for k in names[1::2]}, os.path.join(path, "model-00002-of-00002.safetensors"))
     model, _, _ = load_model(path, torch.float32, "cpu")
     assert torch.equal(model.embed_weight, w["model.embed_tokens.weight"])
+    # a folder whose index names a file that is not there says which file (reference atomserve/loader.py:28-40,
+    # tests/test_cli.py:54-75), not which tensors
+    shards = {k: f"model-0000{1 + i % 2}-of-00002.safetensors" for i, k in enumerate(names)}
+    with open(os.path.join(path, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": shards}, f)
+    load_model(path, torch.float32, "cpu")
+    os.remove(os.path.join(path, "model-00002-of-00002.safetensors"))
+    with pytest.raises(FileNotFoundError, match="lacks model-00002-of-00002.safetensors"):
+        load_model(path, torch.float32, "cpu")
 
 
 def test_a_checkpoint_of_another_layout_is_a_matter_of_the_map_alone():
