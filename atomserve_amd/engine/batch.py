@@ -67,13 +67,14 @@ class RowSplit:
     short_tokens [Ns] int32: the tokens of rows with at most `short` tokens, those that see most keys first;
     long_tiles [Nt, 4] int32: (first flat token, count, row, first position) per `tile` consecutive tokens
     of longer rows, those that see most keys first; max_short_context: host bound on the context of a
-    short token."""
+    short token; tile_keys: the keys that the tiles' last tokens see, added up (what the tiles' attention
+    has to walk: a kernel may choose by it how to cut its work)."""
 
     def __init__(self, short: int, tile: int):
         if short < 0 or tile < 1:
             raise ValueError(f"a row split is (short >= 0, tile >= 1), not {(short, tile)}")
         self.short, self.tile = short, tile
-        self.tokens, self.tiles, self.max_short_context = [], [], 0
+        self.tokens, self.tiles, self.max_short_context, self.tile_keys = [], [], 0, 0
         self.short_tokens = self.long_tiles = None  # on the device once the step is packed
         self.num_short_tokens = self.num_long_tiles = 0
 
@@ -147,6 +148,7 @@ class StepBatch:
                 else:
                     for q0 in range(0, n, split.tile):
                         split.tiles.append((flat + q0, min(split.tile, n - q0), r, row.start + q0))
+                        split.tile_keys += row.start + min(n, q0 + split.tile)
             self.max_context = max(self.max_context, end)
             row_first.append(flat)
             row_len.append(n)

@@ -5,6 +5,7 @@ contiguity, shapes) and only then launches on torch's current stream.  Nothing h
 computes with torch operators: if a library is missing the call raises.
 """
 
+import functools
 import math
 
 import torch
@@ -372,6 +373,8 @@ def attn_decode_fresh(qkv, q_weight, k_weight, cos_sin, slots, eps, store_kv, k_
          _ptr(order) if order is not None else 0, T,
          _ptr(positions), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
          _ptr(part_acc), H, KV, D, bs, float(scale), int(window), part_size, P, _stream())  # fmt: skip
+
+
 PREFILL_TILE_QUERIES = 64  # queries of one work item of the prefill kernel
 PREFILL_MAX_HEAD_DIM = 256  # four stages of 32 keys and values of such heads fill 128 KB of LDS
 
@@ -383,51 +386,99 @@ def attn_prefill_supported(dtype, head_dim: int, block_size: int) -> bool:
 
 # The prefill attention has two variants: a wave owns 32 queries of a head (two column tiles of 16), four waves two
 # heads' 64 queries; or a wave owns 16 and four waves one head's 64, which makes twice the workgroups with half the
-# arithmetic each for the same keys and values brought into LDS.  The second pays while the first would give a
-# compute unit one workgroup at most (a 2,048-token prompt of Qwen3-0.6B sizes 6.24 -> 5.79 ms, 8,192 tokens 30.96 ->
-# 28.27 ms, 512 tokens of Qwen3-8B sizes 11.26 -> 10.92 ms); beyond that it loses (2,048 tokens of Qwen3-8B
-# sizes 28.18 -> 28.28 ms, 16,384 tokens 297.6 -> 323.2 ms).
-PREFILL_QUERY_TILES = None  # 1 or 2 to force a variant (measurements); None: chosen by the sizes
+# arithmetic each for the same keys and values brought into LDS.  And a step of few work items lasts as long as its
+# longest (a portion of 512 tokens behind 15,872 cached ones is 128 workgroups of 256 rounds of 64 keys on a GPU with
+# places for 512): every item may come as several workgroups, the items of more rounds than a piece has cut along
+# their keys into such pieces and merged by a second kernel (csrc/attention.hip, PrefillSplit).
+#
+# Which of the two and how many pieces is chosen by a cost in microseconds, fitted to the kernel's times on 96 steps
+# (portions of 64 to 4,096 tokens behind 0 to 15,872 cached ones, lone prompts of 128 to 16,384 tokens; 16, 32, 40 and
+# 64 heads of 128 on 8 kv heads; 256 compute units; keys and values of 24 layers in turn, so that they come from
+# memory): a round costs a workgroup of the first kind 1.5 us when it has a compute unit to itself and 2.2 us when it
+# shares one, of the second kind 1.25 and 1.4 us; workgroups beyond the places wait for one, in whole turns when the
+# items are equally long and evenly when they are of every length (a lone prompt: one round up to all); the merge
+# costs 6 us and what it writes and reads.  What the cost picks is within 1 per cent of the best of the 12 choices on
+# average there and 22 per cent at worst (the rule it replaces, cut only while pieces x items fit the places and 16
+# queries to a wave only while the workgroups are fewer than the compute units: 2.6 per cent and 38; 512 tokens
+# behind 15,872 of Qwen3-8B sizes 213 -> 173 us, of Qwen3-14B sizes 337 -> 268).
+PREFILL_QUERY_TILES = None  # 1 or 2 to force a variant (measurements and tests); None: by the cost
+PREFILL_PIECES = None  # a number to force that many pieces (1: none; measurements and tests); None: by the cost
+PREFILL_PIECE_CHOICES = (1, 2, 3, 4, 6, 8)
+PREFILL_MIN_PIECE_ROUNDS = 8  # a piece has at least this many rounds (at 24 rounds in all the merge costs what the cut gains)
 
 
-def _prefill_query_tiles(num_tiles: int, H: int, KV: int) -> int:
-    return 1 if num_tiles * KV * -(-2 * (H // KV) // 4) <= compute_units() else 2
+def _prefill_units(query_tiles: int, group: int) -> int:
+    """Workgroups of four waves that share a tile's queries of one kv head."""
+    return -(-(64 // (16 * query_tiles)) * group // 4)
 
 
-
-# A step of few work items lasts as long as its longest: a portion of 512 tokens behind 3,584 cached ones is 128
-# workgroups of 57 to 64 rounds of 64 keys on a GPU with places for 512.  Where the places allow, every item comes as
-# several workgroups, and the items of more rounds than a piece has are cut along their keys into such pieces, merged
-# by a second kernel (csrc/attention.hip, PrefillSplit).  The merge costs some 10 us, and pieces that outnumber the
-# places wait for one: a lone prompt (items of 1 round up to all, as many as places at 2,048 tokens) is slower cut.
-PREFILL_PIECES = None  # a number to force that many pieces (1: none; measurements and tests); None: by the sizes
-PREFILL_MAX_PIECES = 8
-PREFILL_MIN_PIECE_ROUNDS = 8  # a piece has at least this many rounds ...
-PREFILL_MIN_ROUNDS = 28  # ... and the longest item this many, or nothing is cut (at 24 the merge costs what the cut gains)
-
-
-def _prefill_pieces(num_tiles: int, H: int, KV: int, query_tiles: int, max_context: int, window: int = 0) -> tuple:
-    """(pieces, rounds of a piece) for a prompt step; (1, 0): nothing is cut."""
-    units = -(-(64 // (16 * query_tiles)) * (H // KV) // 4)
-    span = min(max_context, window + 64) if window > 0 else max_context  # the keys that the longest item walks
-    rounds = -(-span // 64)
-    if PREFILL_PIECES is not None:
-        pieces = max(1, min(int(PREFILL_PIECES), rounds // 2))
-    elif rounds < PREFILL_MIN_ROUNDS:
-        pieces = 1
+def _prefill_cost(num_tiles: int, H: int, KV: int, D: int, rounds: int, mean_rounds: float, query_tiles: int,
+                  pieces: int, tokens: int) -> float:  # fmt: skip
+    """Microseconds, roughly, of a prompt step's attention: `num_tiles` tiles of 64 queries, the longest item of
+    `rounds` rounds of 64 keys, the items of `mean_rounds` on average."""
+    group, wide = H // KV, D / 128
+    alone, shared = ((1.5, 2.2) if query_tiles == 2 else (1.25, 1.4))
+    per_cu = 2 if D <= 128 else 1  # the rings of wider heads leave room for one workgroup
+    if per_cu == 1:
+        shared = alone
+    places = per_cu * compute_units()
+    workgroups = num_tiles * KV * _prefill_units(query_tiles, group) * pieces
+    piece_rounds = -(-rounds // pieces)
+    if workgroups <= compute_units():
+        cost = piece_rounds * alone
+    elif workgroups <= places:
+        cost = piece_rounds * shared
     else:
-        places = 2 * compute_units()
-        pieces = min(PREFILL_MAX_PIECES, places // (num_tiles * KV * units), rounds // PREFILL_MIN_PIECE_ROUNDS)
-    return (pieces, -(-rounds // pieces)) if pieces > 1 else (1, 0)
+        work = num_tiles * KV * (64 // (16 * query_tiles)) * group / 4 * pieces  # in full workgroups
+        spread = min(1.0, max(0.0, 2.0 * (1.0 - mean_rounds / rounds)))  # 0: all items as long as the longest; 1: of every length
+        evenly = max(piece_rounds * shared, (work * mean_rounds / pieces / places + 0.5 * piece_rounds) * shared)
+        in_turns = -(-workgroups // places) * piece_rounds * shared
+        cost = spread * evenly + (1.0 - spread) * in_turns
+    cost *= wide
+    if pieces > 1:
+        cost += 6.0 + tokens * H * pieces * D * 8 / 2e6  # partial results written and read at 2 TB/s
+    return cost + 6.0
 
 
-def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context, query_tiles=None) -> None:
+def _prefill_plan(num_tiles: int, H: int, KV: int, D: int, max_context: int, window: int = 0, query_tiles=None,
+                  tile_keys: int = 0) -> tuple:  # fmt: skip
+    """(query tiles of a wave, pieces, rounds of a piece) for a prompt step; pieces 1 (and 0 rounds): nothing is cut.
+    tile_keys: the keys that the tiles' last queries see, added up (0: not known; the tiles are then taken to be one
+    request's last ones).  Every layer of a step asks the same question: the answers are kept."""
+    if query_tiles is None:
+        query_tiles = PREFILL_QUERY_TILES
+    return _prefill_plan_of(num_tiles, H, KV, D, max_context, window, query_tiles, tile_keys, PREFILL_PIECES, compute_units())
+
+
+@functools.lru_cache(maxsize=1024)
+def _prefill_plan_of(num_tiles, H, KV, D, max_context, window, query_tiles, tile_keys, forced_pieces, units) -> tuple:
+    span = min(max_context, window + 64) if window > 0 else max_context  # the keys that the longest item walks
+    rounds = max(1, -(-span // 64))
+    if tile_keys > 0:
+        mean_rounds = min(rounds, max(1.0, tile_keys / num_tiles / 64))
+    else:
+        mean_rounds = max(rounds - num_tiles / 2, rounds / 2)
+    kinds = (2, 1) if query_tiles is None else (int(query_tiles),)
+    if forced_pieces is not None:
+        cuts = (max(1, min(int(forced_pieces), rounds // 2)),)
+    else:
+        cuts = tuple(c for c in PREFILL_PIECE_CHOICES if c == 1 or rounds // c >= PREFILL_MIN_PIECE_ROUNDS)
+    tokens = 64 * num_tiles
+    kind, pieces = min(((k, c) for k in kinds for c in cuts),
+                       key=lambda kc: _prefill_cost(num_tiles, H, KV, D, rounds, mean_rounds, kc[0], kc[1], tokens))  # fmt: skip
+    return (kind, pieces, -(-rounds // pieces)) if pieces > 1 else (kind, 1, 0)
+
+
+def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, max_context, query_tiles=None,
+                 tile_keys: int = 0) -> None:  # fmt: skip
     """Causal attention of prompt portions over the paged cache, bfloat16, on the matrix cores.
 
     tiles [Nt, 4] int32: (first flat token, count <= 64, block-table row, position of the first
     token) of up to 64 consecutive tokens of one request; the keys of these tokens are already in
     the pages.  max_context: host bound on the last position + 1 of any tile.
-    query_tiles: column tiles of 16 queries that a wave owns, 2 or 1; None: chosen here."""
+    query_tiles: column tiles of 16 queries that a wave owns, 2 or 1; None: chosen here.
+    tile_keys: the sum over the tiles of (position of the first token + count), if the caller knows it: how the
+    work is cut is chosen better with it (speed only)."""
     _check(q, "q", BF16, (None, None, None))
     T, H, D = q.shape
     _check(out, "out", BF16, (T, H, D))
@@ -442,13 +493,10 @@ def attn_prefill(q, k_pages, v_pages, tiles, block_tables, out, scale, window, m
         raise KernelError(f"prefill attention: unsupported heads {H}/{KV}, head width {D} or page size {bs}")
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
-    if query_tiles is None:
-        query_tiles = PREFILL_QUERY_TILES or _prefill_query_tiles(tiles.shape[0], H, KV)
-    pieces, piece_rounds = _prefill_pieces(tiles.shape[0], H, KV, query_tiles, max_context, window)
+    query_tiles, pieces, piece_rounds = _prefill_plan(tiles.shape[0], H, KV, D, max_context, window, query_tiles, tile_keys)
     cut = part_ml = part_acc = None
     if pieces > 1:
-        units = -(-(64 // (16 * query_tiles)) * (H // KV) // 4)
-        cut = torch.empty(tiles.shape[0] * KV * units, dtype=I32, device=q.device)
+        cut = torch.empty(tiles.shape[0] * KV * _prefill_units(query_tiles, H // KV), dtype=I32, device=q.device)
         part_ml = torch.empty((T, H, pieces, 2), dtype=F32, device=q.device)
         part_acc = torch.empty((T, H, pieces, D), dtype=F32, device=q.device)
     call("as_attn_prefill_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(tiles), tiles.shape[0],
@@ -463,6 +511,8 @@ SKINNY_TWO_MAX_ROWS, SKINNY_TWO_MAX_K = 32, 4096
 # weights' bytes: at 32 rows of 4096 over 256 workgroups (67 MB) the library's product is faster,
 # with rows of 1024 (17 MB) this one is, by the two kernels it saves beside.
 SKINNY_TWO_MAX_ACT_BYTES = 36 << 20
+
+
 def _workgroups() -> int:
     """Persistent kernels run one workgroup per compute unit."""
     return compute_units()

@@ -145,7 +145,7 @@ class Attention(Mixer):
                                   cache.block_tables, out, s.scale, s.window, rows.max_short_context)  # fmt: skip
         if rows.num_long_tiles:
             ops.attn_prefill(q, cache.k_pages, cache.v_pages, rows.long_tiles, cache.block_tables, out, s.scale,
-                             s.window, step.max_context)  # fmt: skip
+                             s.window, step.max_context, tile_keys=rows.tile_keys)  # fmt: skip
 
 
 register("mixer", "attention", Attention)

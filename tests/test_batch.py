@@ -32,6 +32,7 @@ def test_rows_are_flattened_with_slots_tables_and_tiles():
     long = pack([Row(list(range(70)), 0, [list(range(20)), list(range(20))], []), Row([1] * 9, 64, [list(range(20, 40))] * 2, [])])
     # work items of the prefill kernel, the one that sees most keys first
     assert long.split(ATTENTION).long_tiles.tolist() == [[70, 9, 1, 64], [64, 6, 0, 64], [0, 64, 0, 0]]
+    assert long.split(ATTENTION).tile_keys == 73 + 70 + 64  # the keys that each tile's last token sees, added up
     # a prompt's slots are computed as arrays: the same places as token by token, from the middle of a page on
     table = [(7 * i + 3) % 31 for i in range(30)]  # 30 different pages, in no order
     start = BS + 3

@@ -789,12 +789,13 @@ def test_portions_behind_a_long_prefix_cut_their_attention(tmp_path, monkeypatch
         {"step": 5, "entries": [{"id": "a", "tokens": a[2303:], "want": [0, 96]}], "end": ["a"]},
     ]
     decided = []
-    real = ops._prefill_pieces
-    monkeypatch.setattr(ops, "_prefill_pieces", lambda *args, **kw: decided.append(real(*args, **kw)) or decided[-1])
+    real = ops._prefill_plan
+    monkeypatch.setattr(ops, "_prefill_plan", lambda *args, **kw: decided.append(real(*args, **kw)) or decided[-1])
     replay = make_replay(path, "bfloat16", rc.live_token_bound(steps))
     result = compare(replay, steps, requests, raw, weights, {}, "bfloat16", plain_kwargs={"batched": True})
     assert result.rows == 2 + 15 + 3 + 30 + 2 + 2
-    # every step's attention had its pieces decided, layer by layer; with so few heads even the lone first portion is cut
-    assert len(decided) == len(steps) * raw["num_hidden_layers"] and all(pieces > 1 for pieces, _ in decided[3:])
-    assert len({pieces for pieces, _ in decided}) > 1  # into more pieces where the items are fewer
+    # every step's attention had its cut decided, layer by layer: the lone first portion whole, all behind it in pieces
+    layers = raw["num_hidden_layers"]
+    assert len(decided) == len(steps) * layers
+    assert all(pieces == 1 for _, pieces, _ in decided[:layers]) and all(pieces > 1 for _, pieces, _ in decided[layers:])
     assert replay.manager.num_free == replay.manager.num_blocks
