@@ -101,8 +101,19 @@ class StepBatch:
             raise ValueError("a step needs at least one row")
         bs = block_size
         self.splits = {tuple(key): RowSplit(*key) for key in row_splits}
-        tok, pos, trow, want = [], [], [], []
-        slots = [[] for _ in range(num_paged_groups)]
+        # A prompt's portion is hundreds of tokens: its fields are made as arrays; the single tokens of decoding
+        # requests between such rows gather in lists, which become arrays when the next long row (or the end) comes.
+        fields_of_tokens = 3 + num_paged_groups  # token ids, positions, rows, and a slot per group
+        done = [[] for _ in range(fields_of_tokens)]  # arrays, in the order of the rows
+        few = [[] for _ in range(fields_of_tokens)]  # what the short rows since the last array have added
+
+        def settle():
+            for arrays, values in zip(done, few):
+                if values:
+                    arrays.append(np.asarray(values, dtype=np.int32))
+                    values.clear()
+
+        want = []
         row_first, row_len, row_start, row_slots = [], [], [], []
         widths = [max(1, table_width)] * num_paged_groups
         flat = 0
@@ -113,7 +124,8 @@ class StepBatch:
                 raise ValueError(f"bad row: {n} tokens at position {row.start}")
             if any(not 0 <= w < n for w in row.want):
                 raise ValueError(f"bad row: wanted places {row.want} outside its {n} tokens")
-            if n > 64:  # a prompt: checked and addressed as arrays, not token by token
+            long = n > 64  # a prompt: checked and addressed as arrays, not token by token
+            if long:
                 ids = np.asarray(row.tokens, dtype=np.int64)
                 bad = ids[(ids < 0) | (ids >= vocab_size)].tolist()
             else:
@@ -122,24 +134,32 @@ class StepBatch:
                 raise ValueError(f"token id {bad[0]} is outside the vocabulary of {vocab_size}")
             if len(row.tables) != num_paged_groups:
                 raise ValueError(f"row has {len(row.tables)} block tables, the model has {num_paged_groups} groups")
+            if long:
+                settle()
+                places = np.arange(row.start, end, dtype=np.int64)
+                done[0].append(ids.astype(np.int32))
+                done[1].append(places.astype(np.int32))
+                done[2].append(np.full(n, r, dtype=np.int32))
+            else:
+                few[0].extend(row.tokens)
+                few[1].extend(range(row.start, end))
+                few[2].extend([r] * n)
             for g, table in enumerate(row.tables):
                 if end > len(table) * bs:
                     raise ValueError(f"block table holds {len(table) * bs} slots, need {end}")
                 first_page, last_page = row.start // bs, (end - 1) // bs
                 if any(table[b] == RELEASED for b in range(first_page, last_page + 1)):
                     raise ValueError("block table has given back a page that this row writes")
-                if row.store and n > 64:
-                    places = np.arange(row.start, end, dtype=np.int64)
+                if long and row.store:
                     pages = np.asarray(table[first_page : last_page + 1], dtype=np.int64)
-                    slots[g].extend((pages[places // bs - first_page] * bs + places % bs).tolist())
+                    done[3 + g].append((pages[places // bs - first_page] * bs + places % bs).astype(np.int32))
+                elif long:
+                    done[3 + g].append(np.full(n, -1, dtype=np.int32))
                 elif row.store:
-                    slots[g].extend(table[p // bs] * bs + p % bs for p in range(row.start, end))
+                    few[3 + g].extend(table[p // bs] * bs + p % bs for p in range(row.start, end))
                 else:
-                    slots[g].extend([-1] * n)
+                    few[3 + g].extend([-1] * n)
                 widths[g] = max(widths[g], (end + bs - 1) // bs)
-            tok.extend(row.tokens)
-            pos.extend(range(row.start, end))
-            trow.extend([r] * n)
             want.extend(flat + w for w in row.want)
             for split in self.splits.values():
                 if n <= split.short:
@@ -155,12 +175,14 @@ class StepBatch:
             row_start.append(row.start)
             row_slots.append(row.state_slot)
             flat += n
+        settle()
+        tok, pos, trow, *slots = [arrays[0] if len(arrays) == 1 else np.concatenate(arrays) for arrays in done]
 
         # Work items of the prefill kernel, the ones that see most keys first: the kernel hands
         # them out in this order and pairs the longest with the shortest on a compute unit.
         for split in self.splits.values():
             split.tiles.sort(key=lambda t: -(t[3] + t[1]))
-            split.tokens.sort(key=lambda t: -pos[t])  # single queries too: the longest contexts first
+            split.tokens.sort(key=lambda t: -int(pos[t]))  # single queries too: the longest contexts first
             split.max_short_context = max(split.max_short_context, max_context if split.tokens else 0)
         self.max_context = max(self.max_context, max_context)
         T, R = flat, len(rows)
@@ -170,14 +192,15 @@ class StepBatch:
             arr = np.zeros((R, w), dtype=np.int32)
             for r, row in enumerate(rows):
                 t = row.tables[g][:w]
-                arr[r, : len(t)] = [0 if p == RELEASED else p for p in t]
+                arr[r, : len(t)] = t
+            arr[arr == RELEASED] = 0  # a page that was given back: its place names page 0, which nobody reads there
             tables.append(arr)
 
         # Every token; in a decode step those that see most keys first, the order in which the attention
         # kernel's workgroups take whole contexts (`advance` keeps it: the contexts grow together).
         every = range(T)
         if T == R and T > 1:
-            every = np.argsort(-np.asarray(pos, dtype=np.int64), kind="stable")
+            every = np.argsort(-pos.astype(np.int64), kind="stable")
         fields = [("token_ids", tok), ("positions", pos), ("tok_row", trow), ("logits_rows", want),
                   ("all_tokens", every), ("row_first", row_first), ("row_len", row_len), ("row_start", row_start),
                   ("row_slots", row_slots)]  # fmt: skip
