@@ -122,6 +122,39 @@ class StepBatch:
             n, end = len(row.tokens), row.start + len(row.tokens)
             if n < 1 or row.start < 0:
                 raise ValueError(f"bad row: {n} tokens at position {row.start}")
+            if n == 1 and len(row.tables) == num_paged_groups and all(w == 0 for w in row.want) \
+                    and 0 <= row.tokens[0] < vocab_size:  # fmt: skip
+                # A decoding request's one token, the common row of a step: the same checks and entries as
+                # below, without their loops.
+                start, page_at = row.start, row.start // bs
+                for g, table in enumerate(row.tables):
+                    if end > len(table) * bs:
+                        raise ValueError(f"block table holds {len(table) * bs} slots, need {end}")
+                    if table[page_at] == RELEASED:
+                        raise ValueError("block table has given back a page that this row writes")
+                    few[3 + g].append(table[page_at] * bs + start % bs if row.store else -1)
+                    if page_at >= widths[g]:
+                        widths[g] = page_at + 1
+                few[0].append(row.tokens[0])
+                few[1].append(start)
+                few[2].append(r)
+                want.extend([flat] * len(row.want))
+                for split in self.splits.values():
+                    if split.short >= 1:
+                        split.tokens.append(flat)
+                        if end > split.max_short_context:
+                            split.max_short_context = end
+                    else:
+                        split.tiles.append((flat, 1, r, start))
+                        split.tile_keys += end
+                if end > self.max_context:
+                    self.max_context = end
+                row_first.append(flat)
+                row_len.append(1)
+                row_start.append(start)
+                row_slots.append(row.state_slot)
+                flat += 1
+                continue
             if any(not 0 <= w < n for w in row.want):
                 raise ValueError(f"bad row: wanted places {row.want} outside its {n} tokens")
             long = n > 64  # a prompt: checked and addressed as arrays, not token by token
