@@ -1002,32 +1002,6 @@ def test_long_items_of_a_prompt_step_are_cut_into_pieces_and_merged(ops, H, KV, 
         assert torch.allclose(out.float(), whole.float(), atol=2e-2, rtol=2e-2)  # every token, against the kernel without the cut
 
 
-def test_what_the_sizes_say_about_cutting_prompt_steps(ops):
-    """How a prompt step's attention is cut is chosen by a cost fitted to the kernel's times (on 256 compute units,
-    which the costs below assume).  A portion behind a long prefix is few long items: cut along the keys, into the
-    more pieces the fewer the items, a wave owning 32 queries where that still fills the GPU and 16 where only
-    that does.  A lone prompt, a short context, a window that keeps every item short: not cut."""
-    if ops.compute_units() != 256:
-        pytest.skip("the vectors are for 256 compute units")
-    tiles_of = lambda tokens: -(-tokens // 64)
-    plan = lambda tokens, H, context, **kw: ops._prefill_plan(tiles_of(tokens), H, 8, 128, context, **kw)
-    assert plan(512, 32, 16384) == (2, 4, 64)  # 128 items of 256 rounds: four pieces of 64 fill the 512 places
-    assert plan(1024, 32, 16384) == (2, 2, 128)
-    assert plan(512, 16, 16384) == (2, 8, 32)  # half the heads: twice the pieces
-    assert plan(64, 32, 20000) == (1, 8, 40)  # one tile: 16 queries to a wave make twice the workgroups
-    assert plan(512, 32, 4096) == (1, 2, 32)
-    for tokens in (256, 512, 1024, 2048, 4096, 8192, 16384):  # lone prompts: whole
-        assert plan(tokens, 32, tokens)[1:] == (1, 0) and plan(tokens, 16, tokens)[1:] == (1, 0)
-    assert plan(1024, 32, 1024)[0] == 1 and plan(8192, 32, 8192)[0] == 2  # 16 queries to a wave while the workgroups are few
-    assert plan(512, 32, 1024)[1:] == (1, 0)  # 16 rounds: too short to pay for the merge
-    assert plan(512, 32, 8192, window=512)[1:] == (1, 0)  # a window keeps every item short
-    # as many items as places: whole if all are as long as the longest, cut if most are short (`tile_keys` says which)
-    assert plan(2048, 32, 16384, tile_keys=32 * 16384)[1] == 1 and plan(2048, 32, 16384, tile_keys=32 * 4000)[1] > 1
-    # forced for measurements and tests
-    with prefill_cut(ops, 3):
-        assert plan(512, 32, 4096, query_tiles=2) == (2, 3, 22) and plan(512, 32, 100)[1:] == (1, 0)
-
-
 def test_kernels_refuse_what_they_cannot_do(ops):
     from atomserve_amd.kernels.lib import KernelError
 
